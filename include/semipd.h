@@ -871,6 +871,71 @@ int64_t semipd_min_gru_workspace(int64_t num_tokens, int64_t batch, int width);
 int semipd_router_logits(const void* hidden, int64_t ld, const float* weight, float* out, int64_t num_tokens, int width,
                          int num_experts, int dtype, void* stream);
 
+/* ------------------------------------------------------------------ */
+/* RMS norm on an fp32 stream, hashed bigram embedding, latent          */
+/* attention, gated delta rule, clamped gated activation, sigmoid top-k */
+/* ------------------------------------------------------------------ */
+/* stream (fp32 rows, in place) += y when y is given (rows fp32 if y_is_f32, else of `dtype`); when out is given:
+ * out <- stream / sqrt(mean(stream^2) + eps) * (weight + weight_shift) in `dtype` (weight_shift 1: a weight stored around
+ * zero).  Strides in elements.  No reference counterpart. */
+int semipd_rms_stream(const void* y, int64_t y_ld, int y_is_f32, float* stream, int64_t stream_ld, const void* weight,
+                      float weight_shift, float eps, void* out, int64_t out_ld, int64_t rows, int64_t width, int dtype,
+                      void* stream_handle);
+/* out[t] (fp32 [num_tokens, width]) = embed[ids[t]] * scale + bigram[row], row = (previous token * mul_prev + ids[t] *
+ * mul_cur) mod buckets, or `buckets` (the table's last row) for the first token of a sequence.  The token in front of a
+ * request's rows is prev[state_indices[b] * prev_ld] (int32); the call leaves the last token of the request's rows there.
+ * Batch description as in semipd_local_attention.  No reference counterpart. */
+int semipd_embed_bigram(const int64_t* ids, const void* embed, const void* bigram, float scale, int64_t mul_prev,
+                        int64_t mul_cur, int64_t buckets, int32_t* prev, int64_t prev_ld, const int64_t* state_indices,
+                        const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len, int64_t batch,
+                        int64_t num_tokens, float* out, int64_t width, int dtype, void* stream);
+/* Latent attention, the step behind the projection GEMM.  Row t of proj: per head [dim unrotated | rot_dim rotated] query
+ * elements from column 0; at column c_off the latent [rank] and one rotated key part [rot_dim].  pool[loc[t]] <-
+ * [rms_norm(latent) * norm_weight | key part turned]; q_out[t, h * q_head_stride + q_head_off ...) <- head h's rotated part
+ * turned (q_out may be proj itself: in place) (neighbouring pairs of the first rot_dims elements by positions[t] * freq[i], cos and sin times mscale; fp32). */
+int semipd_latent_prep(const void* proj, int64_t ld, int64_t num_tokens, int num_heads, int dim, int rot_dim, int rank,
+                       int64_t c_off, const void* norm_weight, float eps, const int64_t* positions, const float* freq,
+                       int rot_dims, float mscale, void* pool, int64_t pool_ld, const int64_t* loc, void* q_out,
+                       int64_t q_ld, int q_head_stride, int q_head_off, int dtype, void* stream);
+/* Causal softmax attention (+ exp(sink[h]) in the denominator) of num_heads queries [rank + rot_dim] per token over pool
+ * rows [rank + rot_dim] found through req_to_token; the value of a row is its first `rank` elements; out [T, heads * rank].
+ * Batch description and `form` as in semipd_local_attention.  n_splits > 1 (decode batches on the matrix-core form): that
+ * many workgroups share a request's keys and leave partial sums in `partial` (fp32 [rows, heads, n_splits, rank + 2]) for a
+ * merge launch. */
+int semipd_latent_attention(const void* q, int64_t q_ld, void* out, int64_t out_ld, const void* pool, int64_t pool_ld,
+                            const int32_t* req_to_token, int64_t req_to_token_stride, const int64_t* req_pool_indices,
+                            const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len, int64_t batch,
+                            int64_t num_tokens, int64_t max_q_len, int num_heads, int rank, int rot_dim, float scale,
+                            const float* sink, int n_splits, float* partial, int form, int dtype, void* stream);
+/* Gated delta rule over per-request state rows.  Row t of proj holds q | k (num_k_heads x k_dim each) | v | gate
+ * (num_heads x v_dim each) | a | b (num_heads each) at the given columns.  q, k, v pass a causal convolution of `taps`
+ * taps per channel (weights [channels, taps], the last column the current token's) and silu; q, k to unit length (q times
+ * k_dim^-1/2); g = exp(-exp(a_log) softplus(a + dt_bias)), beta = sigmoid(b); per head S <- g S, u = beta (v - S^T k),
+ * S <- S + k u^T, o = S^T q; out = o / rms(o) * norm_weight * silu(gate).  S (fp32 [heads, k_dim, v_dim]) and the last
+ * taps - 1 inputs (fp32 [taps - 1, channels], channels q | k | v) live in state / conv_state[state_indices[b]]: read
+ * unless request b's rows start its sequence, written after its last row.  work: fp32 [num_tokens, work_ld], work_ld >=
+ * semipd_delta_rule_work_width.  Batch description as in semipd_local_attention.  No reference counterpart. */
+int semipd_delta_rule(const void* proj, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, int64_t gate_off,
+                      int64_t a_off, int64_t b_off, const void* conv_q, const void* conv_k, const void* conv_v,
+                      const float* a_log, const float* dt_bias, const void* norm_weight, float eps, float* work,
+                      int64_t work_ld, float* state, int64_t state_ld, float* conv_state, int64_t conv_ld,
+                      const int64_t* state_indices, const int64_t* seq_lens, const int32_t* q_start,
+                      const int32_t* q_len, int64_t batch, int64_t num_tokens, int num_heads, int num_k_heads,
+                      int k_dim, int v_dim, int taps, void* out, int64_t out_ld, int dtype, void* stream);
+int64_t semipd_delta_rule_work_width(int num_heads, int num_k_heads, int k_dim, int v_dim);
+/* Rows of `groups` x [gate ff | up ff] -> rows of `groups` x ff: a = min(gate, limit), b = clamp(up, -limit, limit),
+ * y = a * sigmoid(alpha a) * (b + 1); with routing (topk_weights fp32 / topk_ids int32 [rows, topk]) times the weight of
+ * the group's expert for the row's token, 0 if not chosen.  No reference counterpart. */
+int semipd_clamped_glu(const void* x, int64_t x_ld, void* out, int64_t out_ld, int64_t rows, int64_t ff, int groups,
+                       const float* topk_weights, const int32_t* topk_ids, int topk, float limit, float alpha, int dtype,
+                       void* stream);
+/* sigmoid + top-k (ties to the lower index); renormalize: weights divided by their sum + renorm_eps. */
+int semipd_topk_sigmoid(const void* gating, float* topk_weights, int32_t* topk_ids, int64_t num_tokens, int num_experts,
+                        int topk, int renormalize, float renorm_eps, int dtype, void* stream);
+/* x [rows, width] (row stride x_ld) <- x * sigmoid(gate), fp32 arithmetic.  No reference counterpart. */
+int semipd_sigmoid_gate(void* x, int64_t x_ld, const void* gate, int64_t gate_ld, int64_t rows, int64_t width, int dtype,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

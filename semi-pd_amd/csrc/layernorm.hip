@@ -299,6 +299,112 @@ __global__ void __launch_bounds__(256) routed_relu_square_kernel(T* __restrict__
   }
 }
 
+
+// ---- RMS norm around an fp32 residual stream: stream (+)= y;  out = stream / sqrt(mean(stream^2) + eps) * (weight + shift)
+// (shift 1: a weight stored around zero).  A workgroup per row; the row is summed while it is updated and read once more.
+template <typename T, typename TIn>
+__global__ void __launch_bounds__(256) rms_stream_kernel(const TIn* __restrict__ y, int64_t y_ld, float* __restrict__ stream,
+                                                         int64_t s_ld, const T* __restrict__ w, float shift, float eps,
+                                                         T* __restrict__ out, int64_t out_ld, int64_t width) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  float* x = stream + r * s_ld;
+  float q = 0.f;
+  for (int64_t i = threadIdx.x; i < width; i += 256) {
+    float v = x[i];
+    if (y) {
+      v += Elem<TIn>::to_f(y[r * y_ld + i]);
+      x[i] = v;
+    }
+    q += v * v;
+  }
+  if (!out) return;
+  const float rs = 1.0f / sqrtf(block_sum(q, red) / (float)width + eps);
+  for (int64_t i = threadIdx.x; i < width; i += 256)           // (every thread re-reads the elements it wrote itself)
+    out[r * out_ld + i] = Elem<T>::from_f(x[i] * rs * (Elem<T>::to_f(w[i]) + shift));
+}
+
+// ---- token embedding times a scale plus a row of a hashed bigram table, into the fp32 stream.  The previous token of a
+// row that starts its request's portion is the request's entry of `prev` (an int32 column of the state rows); the first
+// token of a sequence takes the table's last row.  The block of a portion's first row also leaves the portion's last token there.
+template <typename T>
+__global__ void __launch_bounds__(256) embed_bigram_kernel(const int64_t* __restrict__ ids, const T* __restrict__ embed,
+                                                           const T* __restrict__ bigram, float scale, int64_t mul_prev,
+                                                           int64_t mul_cur, int64_t buckets, int32_t* prev, int64_t prev_ld,
+                                                           const int64_t* __restrict__ state_indices,
+                                                           const int64_t* __restrict__ seq_lens, const int32_t* __restrict__ q_start,
+                                                           const int32_t* __restrict__ q_len, int64_t batch, float* __restrict__ out,
+                                                           int64_t width) {
+  __shared__ int64_t row_s;
+  const int64_t t = blockIdx.x;
+  if (threadIdx.x == 0) {
+    int b = -1;
+    int64_t li = 0, n = 1, first_pos = 0;
+    if (q_start == nullptr) {
+      b = (int)t;
+      first_pos = seq_lens[b] - 1;
+    } else {
+      for (int r = 0; r < (int)batch; ++r)
+        if (t >= q_start[r] && t < (int64_t)q_start[r] + q_len[r]) {
+          b = r; li = t - q_start[r]; n = q_len[r]; first_pos = seq_lens[r] - n;
+        }
+    }
+    const int64_t tok = ids[t];
+    int64_t row = buckets;
+    if (b >= 0) {
+      int32_t* slot = prev + state_indices[b] * prev_ld;
+      if (first_pos + li > 0) {
+        const int64_t before = li > 0 ? ids[t - 1] : (int64_t)*slot;
+        row = (before * mul_prev + tok * mul_cur) % buckets;
+      }
+      if (li == 0) *slot = (int32_t)ids[t + n - 1];
+    }
+    row_s = row;
+  }
+  __syncthreads();
+  const T* e = embed + ids[t] * width;
+  const T* g = bigram + row_s * width;
+  for (int64_t i = threadIdx.x; i < width; i += 256) out[t * width + i] = Elem<T>::to_f(e[i]) * scale + Elem<T>::to_f(g[i]);
+}
+
+// ---- gated activation with clamps: rows of `groups` x [gate F | up F] -> rows of `groups` x F,
+//     a = min(gate, limit), b = clamp(up, -limit, limit), y = a * sigmoid(alpha a) * (b + 1)
+// times, when routing is given, the routing weight of the group's expert for the row's token (0 if not chosen).
+template <typename T>
+__global__ void __launch_bounds__(256) clamped_glu_kernel(const T* __restrict__ x, int64_t x_ld, T* __restrict__ out, int64_t out_ld,
+                                                          int64_t rows, int64_t ff, int groups, const float* __restrict__ topk_weights,
+                                                          const int32_t* __restrict__ topk_ids, int topk, float limit, float alpha) {
+  const int64_t width = ff * groups, n = rows * width;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / width, c = i - r * width;
+    const int e = (int)(c / ff);
+    const int64_t f = c - (int64_t)e * ff;
+    float wgt = 1.f;
+    if (topk_ids) {
+      wgt = 0.f;
+      for (int k = 0; k < topk; ++k)
+        if (topk_ids[r * topk + k] == e) wgt = topk_weights[r * topk + k];
+    }
+    const T* row = x + r * x_ld + (int64_t)e * 2 * ff;
+    const float a = fminf(Elem<T>::to_f(row[f]), limit);
+    const float b = fminf(fmaxf(Elem<T>::to_f(row[ff + f]), -limit), limit);
+    out[r * out_ld + c] = Elem<T>::from_f(a / (1.0f + expf(-alpha * a)) * (b + 1.0f) * wgt);
+  }
+}
+
+
+// ---- x <- x * sigmoid(gate), element by element in fp32 (rows of one type, any row strides)
+template <typename T>
+__global__ void __launch_bounds__(256) sigmoid_gate_kernel(T* __restrict__ x, int64_t x_ld, const T* __restrict__ gate, int64_t gate_ld,
+                                                           int64_t rows, int64_t width) {
+  const int64_t n = rows * width;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / width, c = i - r * width;
+    const float g = Elem<T>::to_f(gate[r * gate_ld + c]);
+    x[r * x_ld + c] = Elem<T>::from_f(Elem<T>::to_f(x[r * x_ld + c]) / (1.0f + expf(-g)));
+  }
+}
+
 }  // namespace semipd
 
 using namespace semipd;
@@ -413,4 +519,67 @@ extern "C" int semipd_routed_relu_square(void* u, int64_t ld, const float* topk_
                         hipLaunchKernelGGL((routed_relu_square_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (T*)u,
                                            ld, topk_weights, topk_ids, topk, rows, ff, experts));
   return launch_status("routed_relu_square");
+}
+
+
+extern "C" int semipd_rms_stream(const void* y, int64_t y_ld, int y_is_f32, float* stream, int64_t stream_ld, const void* weight,
+                                 float weight_shift, float eps, void* out, int64_t out_ld, int64_t rows, int64_t width, int dtype,
+                                 void* stream_handle) {
+  SEMIPD_CHECK_ARG(rows >= 0 && width > 0, SEMIPD_EINVAL, "rms_stream: bad sizes");
+  if (rows == 0) return 0;
+  SEMIPD_CHECK_ARG(stream && (y || out) && (!out || weight), SEMIPD_EINVAL, "rms_stream: null pointer");
+  SEMIPD_DISPATCH_DTYPE(dtype, T, {
+    if (y_is_f32)
+      hipLaunchKernelGGL((rms_stream_kernel<T, float>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream_handle),
+                         (const float*)y, y_ld, stream, stream_ld, (const T*)weight, weight_shift, eps, (T*)out, out_ld, width);
+    else
+      hipLaunchKernelGGL((rms_stream_kernel<T, T>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream_handle), (const T*)y, y_ld,
+                         stream, stream_ld, (const T*)weight, weight_shift, eps, (T*)out, out_ld, width);
+  });
+  return launch_status("rms_stream");
+}
+
+extern "C" int semipd_embed_bigram(const int64_t* ids, const void* embed, const void* bigram, float scale, int64_t mul_prev,
+                                   int64_t mul_cur, int64_t buckets, int32_t* prev, int64_t prev_ld, const int64_t* state_indices,
+                                   const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len, int64_t batch,
+                                   int64_t num_tokens, float* out, int64_t width, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && batch >= 0 && width > 0 && buckets > 0, SEMIPD_EINVAL, "embed_bigram: bad sizes");
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(ids && embed && bigram && prev && state_indices && seq_lens && out, SEMIPD_EINVAL, "embed_bigram: null pointer");
+  SEMIPD_CHECK_ARG((q_start == nullptr) == (q_len == nullptr) && (q_start != nullptr || num_tokens == batch), SEMIPD_EINVAL,
+                   "embed_bigram: q_start and q_len come together; without them one row per request");
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((embed_bigram_kernel<T>), dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream), ids,
+                                           (const T*)embed, (const T*)bigram, scale, mul_prev, mul_cur, buckets, prev, prev_ld,
+                                           state_indices, seq_lens, q_start, q_len, batch, out, width));
+  return launch_status("embed_bigram");
+}
+
+extern "C" int semipd_clamped_glu(const void* x, int64_t x_ld, void* out, int64_t out_ld, int64_t rows, int64_t ff, int groups,
+                                  const float* topk_weights, const int32_t* topk_ids, int topk, float limit, float alpha, int dtype,
+                                  void* stream) {
+  SEMIPD_CHECK_ARG(rows >= 0 && ff > 0 && groups > 0 && x_ld >= 2 * ff * groups && out_ld >= ff * groups, SEMIPD_EINVAL,
+                   "clamped_glu: bad sizes");
+  if (rows == 0) return 0;
+  SEMIPD_CHECK_ARG(x && out && ((topk_weights == nullptr) == (topk_ids == nullptr)) && (!topk_ids || topk > 0), SEMIPD_EINVAL,
+                   "clamped_glu: null pointer, or routing weights without ids");
+  const int64_t n = rows * ff * groups;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((clamped_glu_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (const T*)x, x_ld,
+                                           (T*)out, out_ld, rows, ff, groups, topk_weights, topk_ids, topk, limit, alpha));
+  return launch_status("clamped_glu");
+}
+
+extern "C" int semipd_sigmoid_gate(void* x, int64_t x_ld, const void* gate, int64_t gate_ld, int64_t rows, int64_t width, int dtype,
+                                   void* stream) {
+  SEMIPD_CHECK_ARG(rows >= 0 && width > 0 && x_ld >= width && gate_ld >= width, SEMIPD_EINVAL, "sigmoid_gate: bad sizes");
+  if (rows == 0) return 0;
+  SEMIPD_CHECK_ARG(x && gate, SEMIPD_EINVAL, "sigmoid_gate: null pointer");
+  const int64_t n = rows * width;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((sigmoid_gate_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (T*)x, x_ld,
+                                           (const T*)gate, gate_ld, rows, width));
+  return launch_status("sigmoid_gate");
 }

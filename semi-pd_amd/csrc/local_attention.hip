@@ -278,6 +278,67 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_vec_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------------ latent attention: preparation
+// Rows of `proj` hold, per head, [D unrotated | P rotated] query elements from column 0 and, at column c_off, the latent
+// [R] and one rotated key part [P] shared by all heads.  One workgroup per token:
+//   latent / sqrt(mean(latent^2) + eps) * weight -> pool row [0, R); the key part, its first rot_dims elements turned
+//   in neighbouring pairs by position * freq[i] (cos and sin times `mscale`) -> pool row [R, R + P);
+//   the rotated part of every head's query, turned the same way -> q_out[t, h * q_head_stride + q_head_off ...): behind
+//   the R elements that the query times the key up-projection fills, or in place.
+// Angles, the norm and the products are fp32; one rounding on the way out.
+template <typename T>
+__global__ void __launch_bounds__(256) latent_prep_kernel(const T* __restrict__ proj, int64_t ld, int64_t num_tokens, int H, int D,
+                                                          int P, int R, int64_t c_off, const T* __restrict__ norm_w, float eps,
+                                                          const int64_t* __restrict__ positions, const float* __restrict__ freq,
+                                                          int rot_dims, float mscale, T* __restrict__ pool, int64_t pool_ld,
+                                                          const int64_t* __restrict__ loc, T* __restrict__ q_out, int64_t q_ld,
+                                                          int q_head_stride, int q_head_off) {
+  // a workgroup per token: the token's cosines and sines once into LDS for the key part and every head, wave 0 norms the
+  // latent meanwhile, then all threads walk the (unit, pair) items
+  extern __shared__ float cs_l[];          // [rot_dims / 2][2]
+  __shared__ float rs_l;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t t = blockIdx.x;
+  const float pos = (float)positions[t];
+  const int half = rot_dims >> 1;
+  const T* c = proj + t * ld + c_off;
+  T* row = pool + loc[t] * pool_ld;
+  if (wave == 0) {
+    float sq = 0.f;
+    for (int i = lane; i < R; i += 64) {
+      const float v = Elem<T>::to_f(c[i]);
+      sq += v * v;
+    }
+    sq = wave_sum(sq);
+    if (lane == 0) rs_l = 1.0f / sqrtf(sq / (float)R + eps);
+  } else {
+    for (int i = tid - 64; i < half; i += 192) {
+      float sn, cs;
+      sincosf(pos * freq[i], &sn, &cs);
+      cs_l[2 * i] = cs * mscale;
+      cs_l[2 * i + 1] = sn * mscale;
+    }
+  }
+  __syncthreads();
+  const float rs = rs_l;
+  for (int i = tid; i < R; i += 256) row[i] = Elem<T>::from_f(Elem<T>::to_f(c[i]) * rs * Elem<T>::to_f(norm_w[i]));
+  // unit 0: the shared key part behind the latent in the pool row; unit 1 + h: head h's rotated query part
+  const int per = half + (P - rot_dims);             // items of a unit: the pairs, then the elements that pass unchanged
+  for (int item = tid; item < (H + 1) * per; item += 256) {
+    const int u = item / per, i = item % per;
+    const T* src = u == 0 ? c + R : proj + t * ld + (int64_t)(u - 1) * (D + P) + D;
+    T* dst = u == 0 ? row + R : q_out + t * q_ld + (int64_t)(u - 1) * q_head_stride + q_head_off;
+    if (i < half) {
+      const float cs = cs_l[2 * i], sn = cs_l[2 * i + 1];
+      const float x1 = Elem<T>::to_f(src[2 * i]), x2 = Elem<T>::to_f(src[2 * i + 1]);
+      dst[2 * i] = Elem<T>::from_f(x1 * cs - x2 * sn);
+      dst[2 * i + 1] = Elem<T>::from_f(x2 * cs + x1 * sn);
+    } else {
+      dst[rot_dims + (i - half)] = src[rot_dims + (i - half)];
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ shared pieces
 struct LocalAttnArgs {
   const void* q; int64_t q_ld;
@@ -297,6 +358,9 @@ struct LocalAttnArgs {
   const float* head_bias;          // sigmoid weights: added to the score of every key of the head (may be NULL)
   int sigmoid;                     // 0: softmax over the visible keys (+ sink); 1: independent sigmoid weights
   float out_scale;
+  int64_t k_ld, v_ld;              // elements between the rows of two slots (G * D and G * E for pools of their own)
+  int n_splits;                    // decode form: workgroups that share the keys of one (request, kv head, 16 q heads) (0 / 1: one)
+  float* partial;                  // [rows, H, n_splits, E + 2] fp32: unnormalised sums, running maximum, denominator
 };
 
 // first visible position of the contiguous range that ends at the query (the kept first positions come on top)
@@ -334,9 +398,9 @@ __device__ __forceinline__ bool locate_row(const LocalAttnArgs& a, int64_t t, in
 }
 
 // ------------------------------------------------------------------------------------------------ one wave per row
-template <typename T>
+template <typename T, int NA>      // head sizes up to 64 * NA
 __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs a) {
-  __shared__ float q_lds[4][512];
+  __shared__ float q_lds[4][64 * NA];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t t = (int64_t)blockIdx.x * 4 + wave;
   const int h = blockIdx.y;
@@ -355,7 +419,9 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
   const T* vp = (const T*)a.v_pool;
   const bool sig = a.sigmoid != 0;
   const float hb = (sig && a.head_bias) ? a.head_bias[h] : 0.f;
-  float m = sig ? 0.f : -INFINITY, l = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float m = sig ? 0.f : -INFINITY, l = 0.f, acc[NA];
+#pragma unroll
+  for (int u = 0; u < NA; ++u) acc[u] = 0.f;
   constexpr int V = Elem<T>::kVec;
   // the kept first positions (none without a window), then the range that ends at the query
   for (int seg = n_first > 0 ? 0 : 1; seg < 2; ++seg) {
@@ -366,7 +432,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
       const int slot = valid ? row[j] : 0;
       float s = -INFINITY;
       if (valid) {
-        const T* k = kp + ((int64_t)slot * G + g) * D;
+        const T* k = kp + (int64_t)slot * a.k_ld + (int64_t)g * D;
         float dot = 0.f;
         if ((D % V) == 0) {
           for (int d = 0; d < D; d += V) {
@@ -388,16 +454,16 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
         p = valid ? expf(s - m_new) : 0.f;
         l = l * alpha + wave_sum(p);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc[u] *= alpha;
+        for (int u = 0; u < NA; ++u) acc[u] *= alpha;
         m = m_new;
       }
       const int n = (int)((j_last - j0 + 1) < 64 ? (j_last - j0 + 1) : 64);
       for (int jj = 0; jj < n; ++jj) {
         const float pj = __shfl(p, jj, 64);
         const int sj = __shfl(slot, jj, 64);
-        const T* v = vp + ((int64_t)sj * G + g) * E;
+        const T* v = vp + (int64_t)sj * a.v_ld + (int64_t)g * E;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < NA; ++u) {
           const int e = lane + 64 * u;
           if (e < E) acc[u] += pj * Elem<T>::to_f(v[e]);
         }
@@ -409,7 +475,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
   T* o = (T*)a.out + t * a.out_ld + (int64_t)h * E;
   const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)h * E : nullptr;
 #pragma unroll
-  for (int u = 0; u < 8; ++u) {
+  for (int u = 0; u < NA; ++u) {
     const int e = lane + 64 * u;
     if (e < E) {
       float y = acc[u] * inv;
@@ -736,12 +802,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
   const int64_t n_first = keep < blk_lo ? keep : blk_lo;
   if (n_first > 0)
     key_walk<T, ND, NE, 256, true, SIG>(
-        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
-        (int64_t)G * E, row, 0, n_first - 1, 32, v_lds, tid, a.scale, a.cap, [&](int64_t j) { return q_ok && j < n_first; },
+        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+        a.v_ld, row, 0, n_first - 1, 32, v_lds, tid, a.scale, a.cap, [&](int64_t j) { return q_ok && j < n_first; },
         [&](int64_t) { return wave_on; }, r, g, nullptr, 0, hb);
   key_walk<T, ND, NE, 256, true, SIG>(
-      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
-      (int64_t)G * E, row, blk_lo, blk_hi, 32, v_lds, tid, a.scale, a.cap,
+      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+      a.v_ld, row, blk_lo, blk_hi, 32, v_lds, tid, a.scale, a.cap,
       [&](int64_t j) { return q_ok && j <= my_pos && (j >= my_lo || j < keep); },
       [&](int64_t j0) { return wave_on && j0 <= w_hi && (j0 + 31 >= w_lo || j0 < keep); }, r, g, nullptr, blk_lo, hb);
   float l = st.l;
@@ -795,13 +861,24 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
   const int b = blockIdx.x, gk = blockIdx.y;
   const int D = a.D, E = a.E, G = a.G, nd = D >> 5, ne = E >> 4;
   const int rep = a.H / G;
-  const int col0 = blockIdx.z * 16;
+  const int n_splits = a.n_splits > 1 ? a.n_splits : 1, head_groups = (rep + 15) / 16;
+  const int split = blockIdx.z / head_groups;
+  const int col0 = (blockIdx.z % head_groups) * 16;
   const bool col_ok = col0 + r < rep;
   const int h = gk * rep + (col_ok ? col0 + r : col0);
   const int64_t t = a.q_start ? (int64_t)a.q_start[b] + a.q_len[b] - 1 : b;     // the request's newest row
-  const int64_t pos = a.seq_lens[b] - 1;
-  if (pos < 0) return;
-  const int64_t lo = range_lo(a, pos), n_first = kept_before(a, lo);
+  const int64_t pos_q = a.seq_lens[b] - 1;
+  if (pos_q < 0) return;
+  const int64_t lo_q = range_lo(a, pos_q), n_first = split == 0 ? kept_before(a, lo_q) : 0;
+  // with several workgroups per (request, kv head, 16 q heads) this one walks a slice of the range (whole 32-key steps; it
+  // may be empty) and leaves unnormalised sums for the merge kernel
+  int64_t lo = lo_q, pos = pos_q;
+  if (n_splits > 1) {
+    int64_t chunk = (pos_q - lo_q + n_splits) / n_splits;
+    chunk = (chunk + 31) / 32 * 32;
+    lo = lo_q + split * chunk;
+    pos = lo + chunk - 1 < pos_q ? lo + chunk - 1 : pos_q;
+  }
   const float hb = (SIG && a.head_bias) ? a.head_bias[h] * kLog2e : 0.f;
   Frag16 qf[ND];
   {
@@ -825,15 +902,16 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
     for (int64_t j = lo + tid; j <= pos; j += 64 * NW) idx_lds[j - lo] = row[j];
     __syncthreads();
   }
+  // (pos < lo: an empty slice; the walk below does nothing and the partial sums are those of no keys)
   // the kept first positions in front of the window (none without one), then the range that ends at the query
   if (n_first > 0)
     key_walk<T, ND, NE, 64, false, SIG>(
-        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
-        (int64_t)G * E, row, (int64_t)32 * wave, n_first - 1, 32 * NW, mine_b, lane, a.scale, a.cap,
+        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+        a.v_ld, row, (int64_t)32 * wave, n_first - 1, 32 * NW, mine_b, lane, a.scale, a.cap,
         [&](int64_t j) { return j < n_first; }, [&](int64_t) { return true; }, r, g, nullptr, 0, hb);
   key_walk<T, ND, NE, 64, false, SIG>(
-      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
-      (int64_t)G * E, row, lo + 32 * wave, pos, 32 * NW, mine_b, lane, a.scale, a.cap, [&](int64_t j) { return j <= pos; },
+      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+      a.v_ld, row, lo + 32 * wave, pos, 32 * NW, mine_b, lane, a.scale, a.cap, [&](int64_t j) { return j <= pos; },
       [&](int64_t) { return true; }, r, g, idx_fits ? idx_lds : nullptr, lo, hb);
   float l = st.l;
   l += __shfl_xor(l, 16, 64);
@@ -866,6 +944,20 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
     lt += f[w] * part_ml[w][1][c];
   }
   const int hh = gk * rep + col0 + c;
+  if (n_splits > 1) {
+    float* part = a.partial + ((t * a.H + hh) * n_splits + split) * (int64_t)(E + 2);
+    for (int e = slice; e < E; e += 4 * NW) {
+      float y = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) y += f[w] * reinterpret_cast<const float*>(v_lds + w * tile_bytes)[e * 17 + c];
+      part[e] = y;
+    }
+    if (slice == 0) {
+      part[E] = m;
+      part[E + 1] = lt;
+    }
+    return;
+  }
   if (!SIG && a.sink != nullptr) lt += __builtin_amdgcn_exp2f(a.sink[hh] * kLog2e - m);
   const float inv = SIG ? a.out_scale : a.out_scale / lt;
   T* o = (T*)a.out + t * a.out_ld + (int64_t)hh * E;
@@ -874,6 +966,38 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
     float y = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) y += f[w] * reinterpret_cast<const float*>(v_lds + w * tile_bytes)[e * 17 + c];
+    y *= inv;
+    if (gt) y *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * Elem<T>::to_f(gt[e])));
+    o[e] = Elem<T>::from_f(y);
+  }
+}
+
+// The slices of a decode row's keys, each with its own running maximum (base-2 domain), denominator and unnormalised sums:
+// out = sum_s 2^(m_s - m) y_s / (sum_s 2^(m_s - m) l_s + 2^(sink log2 e - m)), a workgroup per (row, head).
+template <typename T, bool SIG>
+__global__ void __launch_bounds__(64) local_attention_merge_kernel(LocalAttnArgs a) {
+  const int64_t b = blockIdx.x;
+  const int h = blockIdx.y, E = a.E, n = a.n_splits;
+  const int64_t t = a.q_start ? (int64_t)a.q_start[b] + a.q_len[b] - 1 : b;
+  if (a.seq_lens[b] - 1 < 0) return;
+  const float* part = a.partial + (t * a.H + h) * n * (int64_t)(E + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < n; ++s) m = fmaxf(m, part[s * (E + 2) + E]);
+  float lt = 0.f;
+  for (int s = 0; s < n; ++s) {
+    const float ms = part[s * (E + 2) + E];
+    lt += (ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m)) * part[s * (E + 2) + E + 1];
+  }
+  if (!SIG && a.sink != nullptr) lt += __builtin_amdgcn_exp2f(a.sink[h] * kLog2e - m);
+  const float inv = SIG ? a.out_scale : a.out_scale / lt;
+  T* o = (T*)a.out + t * a.out_ld + (int64_t)h * E;
+  const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)h * E : nullptr;
+  for (int e = threadIdx.x; e < E; e += 64) {
+    float y = 0.f;
+    for (int s = 0; s < n; ++s) {
+      const float ms = part[s * (E + 2) + E];
+      y += (ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m)) * part[s * (E + 2) + e];
+    }
     y *= inv;
     if (gt) y *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * Elem<T>::to_f(gt[e])));
     o[e] = Elem<T>::from_f(y);
@@ -972,10 +1096,12 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
   const int num_q_heads = a.H, num_kv_heads = a.G, qk_dim = a.D, v_dim = a.E;
   SEMIPD_CHECK_ARG(batch >= 0 && num_tokens >= 0, SEMIPD_EINVAL, "local_attention: bad sizes");
   if (batch == 0 || num_tokens == 0) return 0;
+  if (a.k_ld == 0) a.k_ld = (int64_t)num_kv_heads * qk_dim;
+  if (a.v_ld == 0) a.v_ld = (int64_t)num_kv_heads * v_dim;
   SEMIPD_CHECK_ARG(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, SEMIPD_ESHAPE,
                    "local_attention: %d query heads over %d key/value heads", num_q_heads, num_kv_heads);
-  SEMIPD_CHECK_ARG(qk_dim > 0 && qk_dim <= 512 && v_dim > 0 && v_dim <= 512, SEMIPD_ESHAPE,
-                   "local_attention: head sizes %d / %d (at most 512 / 512)", qk_dim, v_dim);
+  SEMIPD_CHECK_ARG(qk_dim > 0 && qk_dim <= 1024 && v_dim > 0 && v_dim <= 1024, SEMIPD_ESHAPE,
+                   "local_attention: head sizes %d / %d (at most 1024 / 1024)", qk_dim, v_dim);
   SEMIPD_CHECK_ARG(q && out && k_pool && v_pool && a.req_to_token && a.req_pool_indices && a.seq_lens, SEMIPD_EINVAL,
                    "local_attention: null pointer");
   SEMIPD_CHECK_ARG((q_start == nullptr) == (q_len == nullptr), SEMIPD_EINVAL, "local_attention: q_start and q_len come together");
@@ -983,7 +1109,7 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
   SEMIPD_CHECK_ARG(a.cap >= 0.f, SEMIPD_EINVAL, "local_attention: bad cap");
   const bool half = dtype == SEMIPD_BF16 || dtype == SEMIPD_F16;
   const bool mfma_ok = half && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
-                       aligned16(v_pool) && aligned16(out) && out_ld % 8 == 0 &&
+                       aligned16(v_pool) && a.k_ld % 8 == 0 && a.v_ld % 8 == 0 && aligned16(out) && out_ld % 8 == 0 &&
                        (gate == nullptr || (aligned16(gate) && gate_ld % 8 == 0));
   SEMIPD_CHECK_ARG(form != 2 || mfma_ok, SEMIPD_ESHAPE, "local_attention: the matrix-core forms do not take this shape or type");
   if (form != 1 && mfma_ok) {
@@ -991,7 +1117,9 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
     const int tile = 32 * v_tile_row_bytes(v_dim);                       // at most 32 * 576 bytes: below the 64 KB default
     const bool sig = a.sigmoid != 0;
     if (q_start == nullptr || max_q_len <= 1) {
-      const dim3 grid((unsigned)batch, (unsigned)num_kv_heads, (unsigned)((num_q_heads / num_kv_heads + 15) / 16));
+      const int n_splits = (a.n_splits > 1 && a.partial != nullptr) ? a.n_splits : 1;
+      a.n_splits = n_splits;
+      const dim3 grid((unsigned)batch, (unsigned)num_kv_heads, (unsigned)((num_q_heads / num_kv_heads + 15) / 16 * n_splits));
       const int merge = v_dim * 17 * 4;
       const int nw = small ? 8 : 4;
       const size_t lds = nw * (size_t)(tile > merge ? tile : merge);      // up to 80 KB: above the 64 KB default
@@ -1018,6 +1146,16 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
       }
 #undef SEMIPD_LA_DEC
       (void)rc;
+      if (n_splits > 1) {
+        const dim3 mgrid((unsigned)batch, (unsigned)num_q_heads);
+        if (dtype == SEMIPD_BF16) {
+          if (sig) hipLaunchKernelGGL((local_attention_merge_kernel<bf16_t, true>), mgrid, dim3(64), 0, as_stream(stream), a);
+          else hipLaunchKernelGGL((local_attention_merge_kernel<bf16_t, false>), mgrid, dim3(64), 0, as_stream(stream), a);
+        } else {
+          if (sig) hipLaunchKernelGGL((local_attention_merge_kernel<f16_t, true>), mgrid, dim3(64), 0, as_stream(stream), a);
+          else hipLaunchKernelGGL((local_attention_merge_kernel<f16_t, false>), mgrid, dim3(64), 0, as_stream(stream), a);
+        }
+      }
       return launch_status("local_attention_decode");
     }
     a.n_tiles = (num_tokens + 63) / 64 + batch;
@@ -1046,9 +1184,55 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
     return launch_status("local_attention_mfma");
   }
   const dim3 grid((unsigned)((num_tokens + 3) / 4), (unsigned)num_q_heads);
-  SEMIPD_DISPATCH_DTYPE(dtype, T,
-                        hipLaunchKernelGGL((local_attention_rows_kernel<T>), grid, dim3(256), 0, as_stream(stream), a));
+  if (qk_dim <= 512 && v_dim <= 512) {
+    SEMIPD_DISPATCH_DTYPE(dtype, T,
+                          hipLaunchKernelGGL((local_attention_rows_kernel<T, 8>), grid, dim3(256), 0, as_stream(stream), a));
+  } else {
+    SEMIPD_DISPATCH_DTYPE(dtype, T,
+                          hipLaunchKernelGGL((local_attention_rows_kernel<T, 16>), grid, dim3(256), 0, as_stream(stream), a));
+  }
   return launch_status("local_attention");
+}
+
+extern "C" int semipd_latent_prep(const void* proj, int64_t ld, int64_t num_tokens, int num_heads, int dim, int rot_dim, int rank,
+                                  int64_t c_off, const void* norm_weight, float eps, const int64_t* positions, const float* freq,
+                                  int rot_dims, float mscale, void* pool, int64_t pool_ld, const int64_t* loc, void* q_out,
+                                  int64_t q_ld, int q_head_stride, int q_head_off, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && num_heads > 0 && dim >= 0 && rot_dim >= 0 && rank > 0, SEMIPD_EINVAL, "latent_prep: bad sizes");
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= rot_dim, SEMIPD_ESHAPE,
+                   "latent_prep: %d rotated elements of a part of %d", rot_dims, rot_dim);
+  SEMIPD_CHECK_ARG(proj && norm_weight && positions && pool && loc && q_out && (freq || rot_dims == 0), SEMIPD_EINVAL,
+                   "latent_prep: null pointer");
+  SEMIPD_CHECK_ARG(c_off >= (int64_t)num_heads * (dim + rot_dim) && ld >= c_off + rank + rot_dim && pool_ld >= rank + rot_dim &&
+                       q_head_stride >= rot_dim && q_head_off >= 0 && q_head_off + rot_dim <= q_head_stride &&
+                       q_ld >= (int64_t)num_heads * q_head_stride,
+                   SEMIPD_EINVAL, "latent_prep: column ranges overlap or leave the row");
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((latent_prep_kernel<T>), dim3((unsigned)num_tokens), dim3(256),
+                                           (size_t)(rot_dims > 0 ? rot_dims : 2) * sizeof(float), as_stream(stream),
+                                           (const T*)proj, ld, num_tokens, num_heads, dim, rot_dim, rank, c_off, (const T*)norm_weight,
+                                           eps, positions, freq, rot_dims, mscale, (T*)pool, pool_ld, loc, (T*)q_out, q_ld, q_head_stride,
+                                           q_head_off));
+  return launch_status("latent_prep");
+}
+
+// Attention of all heads over ONE row per token that holds the latent [R] and the shared rotated key part [P]: a head's query
+// is [its unrotated part times its key up-projection | its rotated part] (R + P elements), the row is the key and its
+// first R elements are the value -- the softmax-with-sink form of the kernels above with one key/value head whose values are
+// a prefix of its keys.
+extern "C" int semipd_latent_attention(const void* q, int64_t q_ld, void* out, int64_t out_ld, const void* pool, int64_t pool_ld,
+                                       const int32_t* req_to_token, int64_t req_to_token_stride, const int64_t* req_pool_indices,
+                                       const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len, int64_t batch,
+                                       int64_t num_tokens, int64_t max_q_len, int num_heads, int rank, int rot_dim, float scale,
+                                       const float* sink, int n_splits, float* partial, int form, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(rank > 0 && rot_dim >= 0 && pool_ld >= rank + rot_dim, SEMIPD_EINVAL, "latent_attention: bad sizes");
+  SEMIPD_CHECK_ARG(n_splits >= 0 && n_splits <= 64 && (n_splits <= 1 || partial != nullptr), SEMIPD_EINVAL,
+                   "latent_attention: up to 64 slices of the keys, with room for their partial sums");
+  LocalAttnArgs a{q, q_ld, nullptr, 0, out, out_ld, pool, pool, req_to_token, req_to_token_stride, req_pool_indices,
+                  seq_lens, q_start, q_len, batch, num_tokens, num_heads, 1, rank + rot_dim, rank, sink, scale, 0.f,
+                  0, 0, 0, 0, nullptr, 0, 1.0f, pool_ld, pool_ld, n_splits, partial};
+  return launch_local_attention(a, max_q_len, form, dtype, stream);
 }
 
 extern "C" int semipd_local_attention_mfma_supported(int num_q_heads, int num_kv_heads, int qk_dim, int v_dim, int dtype) {

@@ -70,7 +70,8 @@ __global__ void __launch_bounds__(64)
 moe_topk_kernel(const T* __restrict__ gating, const float* __restrict__ bias,
                 float* __restrict__ topk_weights, int32_t* __restrict__ topk_ids, int E, int topk,
                 int num_group, int topk_group, int renormalize, int scoring, int grouped,
-                const float* __restrict__ planes = nullptr, int n_planes = 0, int64_t plane_elems = 0) {
+                const float* __restrict__ planes = nullptr, int n_planes = 0, int64_t plane_elems = 0,
+                float renorm_eps = 0.f) {
   constexpr int NE = kMaxExperts / 64;
   __shared__ float choice[kMaxExperts];  // group stage: the selection values of every expert
   __shared__ float gscore[64];
@@ -232,7 +233,7 @@ moe_topk_kernel(const T* __restrict__ gating, const float* __restrict__ bias,
         const float s = Elem<T>::to_f(Elem<T>::from_f(wsum));
         wgt = Elem<T>::to_f(Elem<T>::from_f(my_w / s));
       } else {
-        wgt = my_w / wsum;
+        wgt = my_w / (wsum + renorm_eps);
       }
     }
     topk_weights[t * topk + lane] = wgt;
@@ -594,6 +595,19 @@ int semipd_topk_softmax(const void* gating, float* topk_weights, int32_t* topk_i
   SEMIPD_CHECK_ARG(gating && topk_weights && topk_ids, SEMIPD_EINVAL, "topk_softmax: null pointer");
   SEMIPD_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL((moe_topk_kernel<T>), dim3((unsigned)num_tokens), dim3(64), 0, as_stream(stream), (const T*)gating, (const float*)nullptr, topk_weights, topk_ids, num_experts, topk, 1, 1, renormalize, 0, 0));
   return launch_status("topk_softmax");
+}
+
+// Independent sigmoid scores of all experts, the topk largest kept (ties to the lower index); renormalize: divided by their
+// sum + renorm_eps.
+int semipd_topk_sigmoid(const void* gating, float* topk_weights, int32_t* topk_ids, int64_t num_tokens, int num_experts,
+                        int topk, int renormalize, float renorm_eps, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && num_experts > 0 && num_experts <= kMaxExperts && topk > 0 &&
+                       topk <= kMaxTopk && topk <= num_experts,
+                   SEMIPD_EINVAL, "topk_sigmoid: bad sizes (E<=%d, topk<=%d)", kMaxExperts, kMaxTopk);
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(gating && topk_weights && topk_ids, SEMIPD_EINVAL, "topk_sigmoid: null pointer");
+  SEMIPD_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL((moe_topk_kernel<T>), dim3((unsigned)num_tokens), dim3(64), 0, as_stream(stream), (const T*)gating, (const float*)nullptr, topk_weights, topk_ids, num_experts, topk, 1, 1, renormalize, 1, 0, (const float*)nullptr, 0, (int64_t)0, renorm_eps));
+  return launch_status("topk_sigmoid");
 }
 
 int semipd_grouped_topk(const void* gating, const float* correction_bias, float* topk_weights,

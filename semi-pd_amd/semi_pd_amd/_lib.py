@@ -163,10 +163,22 @@ _SIGNATURES = {
                        _f32, _vp, _i64, _i32, _vp],
     "semipd_min_gru_workspace": [_i64, _i64, _i32],
     "semipd_router_logits": [_vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
+    "semipd_rms_stream": [_vp, _i64, _i32, _vp, _i64, _vp, _f32, _f32, _vp, _i64, _i64, _i64, _i32, _vp],
+    "semipd_embed_bigram": [_vp, _vp, _vp, _f32, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i32, _vp],
+    "semipd_latent_prep": [_vp, _i64, _i64, _i32, _i32, _i32, _i32, _i64, _vp, _f32, _vp, _vp, _i32, _f32, _vp, _i64, _vp, _vp,
+                           _i64, _i32, _i32, _i32, _vp],
+    "semipd_latent_attention": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32,
+                                _i32, _f32, _vp, _i32, _vp, _i32, _i32, _vp],
+    "semipd_delta_rule": [_vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _vp, _i64,
+                          _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _i64, _i32, _vp],
+    "semipd_delta_rule_work_width": [_i32, _i32, _i32, _i32],
+    "semipd_clamped_glu": [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _vp, _vp, _i32, _f32, _f32, _i32, _vp],
+    "semipd_topk_sigmoid": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _i32, _vp],
+    "semipd_sigmoid_gate": [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _vp],
 }
 _RESTYPES = {"semipd_last_error": C.c_char_p, "semipd_lm_head_argmax_workspace": _sz,
              "semipd_linear_workspace": _sz, "semipd_stream_linear_workspace": _sz, "semipd_dense_gemm_report": _sz, "semipd_ar_meta_size": _sz, "semipd_ar_region_size": _sz,
-             "semipd_min_gru_workspace": _i64}
+             "semipd_min_gru_workspace": _i64, "semipd_delta_rule_work_width": _i64}
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
@@ -180,6 +192,7 @@ CORE_SOURCES = ("elementwise.hip", "skinny_gemm.hip", "stream_linear.hip", "gemm
 MODEL_SOURCES = {
     "Kudirax": ("local_attention.hip", "layernorm.hip"),
     "Tigotar": ("local_attention.hip", "layernorm.hip", "recurrent.hip"),
+    "Penozen": ("local_attention.hip", "layernorm.hip", "delta_rule.hip"),
 }
 
 

@@ -1583,3 +1583,212 @@ def router_logits(hidden_states: torch.Tensor, weight: torch.Tensor) -> torch.Te
     check(_lib.load().semipd_router_logits(ptr(hidden_states), hidden_states.stride(0), ptr(weight), ptr(out), T, W, weight.shape[0],
                                            dtype_code(hidden_states.dtype), current_stream(hidden_states.device)), "router_logits")
     return out
+
+
+# ---- RMS norm on an fp32 stream, hashed bigram embedding, latent attention, gated delta rule, clamped gated experts -------
+def rms_stream(y: Optional[torch.Tensor], stream: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
+               weight_shift: float = 0.0, want_out: bool = True) -> Optional[torch.Tensor]:
+    """stream (fp32 [rows, width], in place) += y (rows fp32 or of the weight's type; None: nothing is added); returns
+    stream / sqrt(mean(stream^2) + eps) * (weight + weight_shift) in the weight's type (None with want_out=False)
+    (csrc/layernorm.hip: semipd_rms_stream)."""
+    if stream.dim() != 2 or stream.dtype != torch.float32 or stream.stride(1) != 1:
+        raise RuntimeError("rms_stream: the stream is fp32 [rows, width] with contiguous rows")
+    rows, width = stream.shape
+    if want_out and (weight is None or weight.shape != (width,) or not weight.is_contiguous()):
+        raise RuntimeError("rms_stream: weight is contiguous [width]")
+    if y is None and not want_out:
+        return None
+    dt = weight.dtype if weight is not None else y.dtype
+    if y is not None and (y.shape != stream.shape or y.stride(1) != 1 or y.dtype not in (dt, torch.float32)):
+        raise RuntimeError("rms_stream: y is shaped like the stream, fp32 or of the weight's type")
+    out = torch.empty((rows, width), dtype=dt, device=stream.device) if want_out else None
+    check(_lib.load().semipd_rms_stream(ptr(y), y.stride(0) if y is not None else 0,
+                                        1 if (y is not None and y.dtype == torch.float32 and dt != torch.float32) else 0,
+                                        ptr(stream), stream.stride(0), ptr(weight), float(weight_shift), float(eps), ptr(out),
+                                        out.stride(0) if out is not None else 0, rows, width, dtype_code(dt),
+                                        current_stream(stream.device)), "rms_stream")
+    return out
+
+
+def _batch_rows(name: str, T: int, B: int, q_start, q_len) -> None:
+    if (q_start is None) != (q_len is None) or (q_start is None and T != B):
+        raise RuntimeError(f"{name}: q_start and q_len come together; without them one row per request")
+    if q_start is not None and (q_start.dtype != torch.int32 or q_len.dtype != torch.int32 or q_start.shape[0] != B
+                                or q_len.shape[0] != B):
+        raise RuntimeError(f"{name}: q_start / q_len are int32 [B]")
+
+
+def embed_bigram(input_ids: torch.Tensor, embed: torch.Tensor, bigram: torch.Tensor, scale: float, mul_prev: int, mul_cur: int,
+                 buckets: int, prev_token: torch.Tensor, state_indices: torch.Tensor, seq_lens: torch.Tensor,
+                 q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor]) -> torch.Tensor:
+    """fp32 [T, width] = embed[id] * scale + bigram[(previous id * mul_prev + id * mul_cur) mod buckets] (row `buckets` for the
+    first token of a sequence).  prev_token: int32 [slots, 1] view of the requests' state rows (any row stride): the token
+    in front of a request's rows is read there and the last token of its rows is left there (csrc/layernorm.hip)."""
+    T, B = input_ids.shape[0], state_indices.shape[0]
+    width = embed.shape[1]
+    if input_ids.dtype != torch.int64 or not input_ids.is_contiguous() or embed.dtype != bigram.dtype \
+            or bigram.shape != (buckets + 1, width) or not embed.is_contiguous() or not bigram.is_contiguous():
+        raise RuntimeError("embed_bigram: int64 ids, embed [V, W] and bigram [buckets + 1, W] contiguous and of one type")
+    if prev_token.dtype != torch.int32 or prev_token.dim() != 2 or prev_token.shape[1] < 1:
+        raise RuntimeError("embed_bigram: prev_token is int32 [slots, >= 1]")
+    if state_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64 or seq_lens.shape[0] != B:
+        raise RuntimeError("embed_bigram: state_indices / seq_lens are int64 [B]")
+    _batch_rows("embed_bigram", T, B, q_start, q_len)
+    out = torch.empty((T, width), dtype=torch.float32, device=embed.device)
+    check(_lib.load().semipd_embed_bigram(ptr(input_ids), ptr(embed), ptr(bigram), float(scale), int(mul_prev), int(mul_cur),
+                                          int(buckets), ptr(prev_token), prev_token.stride(0), ptr(state_indices), ptr(seq_lens),
+                                          ptr(q_start), ptr(q_len), B, T, ptr(out), width, dtype_code(embed.dtype),
+                                          current_stream(embed.device)), "embed_bigram")
+    return out
+
+
+def latent_prep(proj: torch.Tensor, num_heads: int, dim: int, rot_dim: int, rank: int, c_off: int, norm_weight: torch.Tensor,
+                eps: float, positions: torch.Tensor, freq: Optional[torch.Tensor], rot_dims: int, mscale: float,
+                pool: torch.Tensor, loc: torch.Tensor, q_out: Optional[torch.Tensor] = None) -> None:
+    """Rows of `proj`: per head [dim | rot_dim] query elements from column 0, the latent [rank] and the shared rotated key
+    part [rot_dim] at column c_off.  pool[loc] <- [rms_norm(latent) * norm_weight | key part turned by the position];
+    q_out [T, heads * (rank + rot_dim)]: every head's last rot_dim elements <- its rotated query part turned; without q_out
+    the rotated query parts are turned in place (csrc/local_attention.hip: semipd_latent_prep)."""
+    T = proj.shape[0]
+    if proj.dim() != 2 or proj.stride(1) != 1:
+        raise RuntimeError("latent_prep: proj is 2-D with contiguous rows")
+    if q_out is None:
+        q_out, stride, off = proj, dim + rot_dim, dim
+    else:
+        stride, off = rank + rot_dim, rank
+        if q_out.dim() != 2 or q_out.stride(1) != 1 or q_out.dtype != proj.dtype or q_out.shape != (T, num_heads * (rank + rot_dim)):
+            raise RuntimeError("latent_prep: q_out is [T, heads * (rank + rot_dim)] of the activation type")
+    if pool.dim() != 2 or pool.dtype != proj.dtype or pool.shape[1] != rank + rot_dim or pool.stride(1) != 1:
+        raise RuntimeError(f"latent_prep: the pool is [N, {rank + rot_dim}] of {proj.dtype}")
+    if loc.dtype != torch.int64 or positions.dtype != torch.int64 or loc.shape[0] != T or positions.shape[0] != T:
+        raise RuntimeError("latent_prep: one int64 pool slot and position per row")
+    if norm_weight.shape != (rank,) or norm_weight.dtype != proj.dtype or not norm_weight.is_contiguous():
+        raise RuntimeError("latent_prep: norm_weight is contiguous [rank] of the activation type")
+    if rot_dims and (freq is None or freq.dtype != torch.float32 or freq.numel() != rot_dims // 2 or not freq.is_contiguous()):
+        raise RuntimeError("latent_prep: freq is fp32 [rot_dims / 2]")
+    check(_lib.load().semipd_latent_prep(ptr(proj), proj.stride(0), T, num_heads, dim, rot_dim, rank, int(c_off), ptr(norm_weight),
+                                         float(eps), ptr(positions), ptr(freq), int(rot_dims), float(mscale), ptr(pool),
+                                         pool.stride(0), ptr(loc), ptr(q_out), q_out.stride(0), stride, off, dtype_code(proj.dtype),
+                                         current_stream(proj.device)), "latent_prep")
+
+
+def latent_attention_fwd(q: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, rank: int, req_to_token: torch.Tensor,
+                         req_pool_indices: torch.Tensor, seq_lens: torch.Tensor, q_start: Optional[torch.Tensor],
+                         q_len: Optional[torch.Tensor], max_q_len: int, sm_scale: float, sink: Optional[torch.Tensor] = None,
+                         form: int = 0, n_splits: int = 1) -> None:
+    """Causal softmax attention (+ exp(sink) in every head's denominator) over pool rows [N, rank + rot_dim] whose first
+    `rank` elements are also the values: q [T, H * (rank + rot_dim)], out [T, H * rank]; batch description as in
+    local_attention_fwd (csrc/local_attention.hip: semipd_latent_attention).  n_splits > 1: a decode batch whose requests'
+    keys are shared out over that many workgroups each (the matrix-core decode form; other forms ignore it)."""
+    T = q.shape[0]
+    width = pool.shape[1]
+    if q.dim() != 2 or out.dim() != 2 or q.stride(1) != 1 or out.stride(1) != 1 or q.shape[1] % width or pool.dim() != 2 \
+            or pool.stride(1) != 1 or not 0 < rank <= width:
+        raise RuntimeError("latent_attention_fwd: q [T, H * row], out [T, H * rank], pool [N, row] with contiguous rows")
+    H = q.shape[1] // width
+    if out.shape != (T, H * rank) or out.dtype != q.dtype or pool.dtype != q.dtype:
+        raise RuntimeError("latent_attention_fwd: shapes or types of q, out and the pool disagree")
+    if sink is not None and (sink.dtype != torch.float32 or sink.numel() != H or not sink.is_contiguous()):
+        raise RuntimeError("latent_attention_fwd: sink is fp32 [H]")
+    if req_to_token.dtype != torch.int32 or req_pool_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64:
+        raise RuntimeError("latent_attention_fwd: req_to_token int32, req_pool_indices / seq_lens int64")
+    B = req_pool_indices.shape[0]
+    _batch_rows("latent_attention_fwd", T, B, q_start, q_len)
+    n_splits = int(n_splits) if (q_start is None and q.dtype != torch.float32) else 1
+    partial = torch.empty((T, H, n_splits, rank + 2), dtype=torch.float32, device=q.device) if n_splits > 1 else None
+    check(_lib.load().semipd_latent_attention(ptr(q), q.stride(0), ptr(out), out.stride(0), ptr(pool), pool.stride(0),
+                                              ptr(req_to_token), req_to_token.stride(0), ptr(req_pool_indices), ptr(seq_lens),
+                                              ptr(q_start), ptr(q_len), B, T, int(max_q_len), H, int(rank), width - int(rank),
+                                              float(sm_scale), ptr(sink), n_splits, ptr(partial), int(form), dtype_code(q.dtype),
+                                              current_stream(q.device)), "latent_attention")
+
+
+def delta_rule(proj: torch.Tensor, offsets, conv_q: torch.Tensor, conv_k: torch.Tensor, conv_v: torch.Tensor, a_log: torch.Tensor,
+               dt_bias: torch.Tensor, norm_weight: torch.Tensor, eps: float, state: torch.Tensor, conv_state: Optional[torch.Tensor],
+               state_indices: torch.Tensor, seq_lens: torch.Tensor, q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor],
+               num_heads: int, num_k_heads: int, k_dim: int, v_dim: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The gated delta rule behind its projection GEMM (csrc/delta_rule.hip).  offsets = columns of q, k, v, gate, a, b in the
+    rows of `proj`; conv_* [channels, taps]; a_log / dt_bias fp32 [H]; state fp32 [slots, H * k_dim * v_dim] and conv_state
+    fp32 [slots, (taps - 1) * channels] are column ranges of the requests' state rows.  Returns [T, H * v_dim]."""
+    T, B = proj.shape[0], state_indices.shape[0]
+    taps = conv_q.shape[1]
+    gd, hv = num_k_heads * k_dim, num_heads * v_dim
+    if proj.dim() != 2 or proj.stride(1) != 1 or len(offsets) != 6:
+        raise RuntimeError("delta_rule: proj is 2-D with contiguous rows; six column offsets")
+    for wt, rows in ((conv_q, gd), (conv_k, gd), (conv_v, hv)):
+        if wt.shape != (rows, taps) or wt.dtype != proj.dtype or not wt.is_contiguous():
+            raise RuntimeError("delta_rule: convolution weights are contiguous [channels, taps] of the activation type")
+    for vec in (a_log, dt_bias):
+        if vec.dtype != torch.float32 or vec.shape != (num_heads,) or not vec.is_contiguous():
+            raise RuntimeError("delta_rule: a_log / dt_bias are fp32 [H]")
+    if norm_weight.shape != (v_dim,) or norm_weight.dtype != proj.dtype or not norm_weight.is_contiguous():
+        raise RuntimeError("delta_rule: norm_weight is contiguous [v_dim] of the activation type")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != num_heads * k_dim * v_dim or state.stride(1) != 1:
+        raise RuntimeError("delta_rule: state is fp32 [slots, H * k_dim * v_dim]")
+    if taps > 1 and (conv_state is None or conv_state.dtype != torch.float32 or conv_state.dim() != 2
+                     or conv_state.shape[1] != (taps - 1) * (2 * gd + hv) or conv_state.stride(1) != 1):
+        raise RuntimeError("delta_rule: conv_state is fp32 [slots, (taps - 1) * channels]")
+    if state_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64 or seq_lens.shape[0] != B:
+        raise RuntimeError("delta_rule: state_indices / seq_lens are int64 [B]")
+    _batch_rows("delta_rule", T, B, q_start, q_len)
+    ends = [offsets[0] + gd, offsets[1] + gd, offsets[2] + hv, offsets[3] + hv, offsets[4] + num_heads, offsets[5] + num_heads]
+    if min(offsets) < 0 or max(ends) > proj.shape[1]:
+        raise RuntimeError("delta_rule: a column range leaves the row")
+    if out is None:
+        out = torch.empty((T, hv), dtype=proj.dtype, device=proj.device)
+    elif out.shape != (T, hv) or out.dtype != proj.dtype or out.stride(1) != 1:
+        raise RuntimeError("delta_rule: out is [T, H * v_dim] of the activation type")
+    lib = _lib.load()
+    wld = int(lib.semipd_delta_rule_work_width(num_heads, num_k_heads, k_dim, v_dim))
+    work = torch.empty((T, wld), dtype=torch.float32, device=proj.device)
+    check(lib.semipd_delta_rule(ptr(proj), proj.stride(0), *[int(o) for o in offsets], ptr(conv_q), ptr(conv_k), ptr(conv_v),
+                                ptr(a_log), ptr(dt_bias), ptr(norm_weight), float(eps), ptr(work), wld, ptr(state), state.stride(0),
+                                ptr(conv_state), conv_state.stride(0) if conv_state is not None else 0, ptr(state_indices),
+                                ptr(seq_lens), ptr(q_start), ptr(q_len), B, T, num_heads, num_k_heads, k_dim, v_dim, taps, ptr(out),
+                                out.stride(0), dtype_code(proj.dtype), current_stream(proj.device)), "delta_rule")
+    return out
+
+
+def clamped_glu(x: torch.Tensor, limit: float, alpha: float, groups: int = 1, topk_weights: Optional[torch.Tensor] = None,
+                topk_ids: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [rows, groups * 2 * ff], every group [gate ff | up ff] -> [rows, groups * ff]: a = min(gate, limit),
+    b = clamp(up, -limit, limit), a * sigmoid(alpha a) * (b + 1); with routing, times the routing weight of the group's
+    expert for the row's token (0 if the token does not use it) (csrc/layernorm.hip: semipd_clamped_glu)."""
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] % (2 * groups):
+        raise RuntimeError("clamped_glu: x is [rows, groups * 2 * ff] with contiguous rows")
+    rows, ff = x.shape[0], x.shape[1] // (2 * groups)
+    if (topk_weights is None) != (topk_ids is None):
+        raise RuntimeError("clamped_glu: routing weights come with their ids")
+    k = 0
+    if topk_ids is not None:
+        if topk_weights.dtype != torch.float32 or topk_ids.dtype != torch.int32 or topk_weights.shape != topk_ids.shape \
+                or topk_ids.shape[0] != rows or not topk_weights.is_contiguous() or not topk_ids.is_contiguous():
+            raise RuntimeError("clamped_glu: topk_weights fp32 / topk_ids int32 [rows, k] contiguous")
+        k = topk_ids.shape[1]
+    out = torch.empty((rows, groups * ff), dtype=x.dtype, device=x.device)
+    check(_lib.load().semipd_clamped_glu(ptr(x), x.stride(0), ptr(out), out.stride(0), rows, ff, groups, ptr(topk_weights),
+                                         ptr(topk_ids), k, float(limit), float(alpha), dtype_code(x.dtype),
+                                         current_stream(x.device)), "clamped_glu")
+    return out
+
+
+def topk_sigmoid(gating_output: torch.Tensor, topk: int, renormalize: bool, renorm_eps: float = 0.0):
+    """Independent sigmoid scores of all experts, the topk largest kept (ties to the lower index) and -- renormalize -- divided
+    by their sum + renorm_eps: (weights fp32 [T, k], ids int32 [T, k])."""
+    T, E = gating_output.shape
+    w = torch.empty((T, topk), dtype=torch.float32, device=gating_output.device)
+    ids = torch.empty((T, topk), dtype=torch.int32, device=gating_output.device)
+    g = gating_output.contiguous()
+    check(_lib.load().semipd_topk_sigmoid(ptr(g), ptr(w), ptr(ids), T, E, topk, int(renormalize), float(renorm_eps),
+                                          dtype_code(g.dtype), current_stream(g.device)), "topk_sigmoid")
+    return w, ids
+
+
+def sigmoid_gate_(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """x <- x * sigmoid(gate) in place, fp32 arithmetic (csrc/layernorm.hip); x and gate [rows, width] of one type, rows may be
+    column ranges of wider rows."""
+    if x.dim() != 2 or x.shape != gate.shape or x.dtype != gate.dtype or x.stride(1) != 1 or gate.stride(1) != 1:
+        raise RuntimeError("sigmoid_gate_: x and gate are [rows, width] of one type with contiguous rows")
+    check(_lib.load().semipd_sigmoid_gate(ptr(x), x.stride(0), ptr(gate), gate.stride(0), x.shape[0], x.shape[1],
+                                          dtype_code(x.dtype), current_stream(x.device)), "sigmoid_gate")
+    return x
