@@ -113,6 +113,7 @@ class HipAttnBackend(AttentionBackend):
         self.model_runner = model_runner
         self._algo = (0.0, 0.0)  # algorithmic (bytes, flops) per layer call of the current batch
         self._fused_decode_ok = {}
+        self._decode_len_bound = self.max_context_len          # how long the requests of the current decode batch can be
 
     @property
     def num_cus(self) -> int:
@@ -130,6 +131,7 @@ class HipAttnBackend(AttentionBackend):
                                              forward_batch.seq_lens, kv_indptr, None, kv_indices)
             max_len = self.max_context_len if forward_batch.seq_lens_sum is None else max(
                 1, forward_batch.seq_lens_sum // max(bs, 1))
+            self._decode_len_bound = max_len
             splits = self.fixed_kv_splits or choose_kv_splits(
                 bs, self.num_kv_head, max_len, self.num_cus, self.num_kv_splits_cap, mla=self.is_mla,
                 mla_heads=self.num_head if self.is_mla else 0)
@@ -174,6 +176,7 @@ class HipAttnBackend(AttentionBackend):
         """Called inside the capture: the kv_indices build kernel is recorded into the graph and reads
         the static req_pool_indices / seq_lens buffers on every replay."""
         assert forward_mode.is_decode()
+        self._decode_len_bound = self.max_context_len          # a captured graph serves every length
         splits = num_kv_splits or self.fixed_kv_splits or choose_kv_splits(bs, self.num_kv_head, self.max_context_len, self.num_cus,
                                                    self.num_kv_splits_cap, mla=self.is_mla,
                                                    mla_heads=self.num_head if self.is_mla else 0)
@@ -298,6 +301,37 @@ class HipAttnBackend(AttentionBackend):
         if kt:
             kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
         return out
+
+    # ---- latent attention: one row per token is key (latent + shared rotated part) and value (the latent) ---------------
+    def forward_latent(self, q, layer, forward_batch: ForwardBatch, sink=None):
+        """Causal softmax attention with a sink term over the pool rows of a latent-attention layer (the model stored them
+        with the step that prepares q): q [T, heads * (rank + rot_dim)] holds, per head, the unrotated query part times the
+        key up-projection and the rotated part; the result [T, heads * rank] is the weighted sum of latents, which the
+        model expands with the value up-projection.  One call for prompt portions, single tokens and decode batches."""
+        T = q.shape[0]
+        rank = layer.v_head_dim
+        o = torch.empty((T, layer.tp_q_head_num * rank), dtype=q.dtype, device=q.device)
+        rows = forward_batch.token_to_kv_pool.get_key_buffer(layer.layer_id)
+        n_splits = 1
+        if forward_batch.forward_mode.is_decode():
+            q_start = q_len = None
+            max_q = 1
+            # all heads of a request share its rows, so a decode batch is only (requests x groups of 16 heads) workgroups:
+            # below two per CU the keys of a request are shared out over several, about 128 keys each at least
+            wgs = T * ((layer.tp_q_head_num + 15) // 16)
+            n_splits = max(1, min(16, (2 * max(1, self.num_cus)) // max(wgs, 1), self._decode_len_bound // 128))
+            n_splits = int(os.environ.get("SEMIPD_LATENT_DECODE_SPLITS", n_splits))
+        else:
+            q_start, q_len = forward_batch.extend_start_loc, forward_batch.extend_seq_lens
+            max_q = max(forward_batch.extend_seq_lens_cpu)
+        kt = self._timing()
+        t0 = kt.start() if kt else None
+        ops.latent_attention_fwd(q, o, rows.view(rows.shape[0], -1), rank, self.req_to_token, forward_batch.req_pool_indices,
+                                 forward_batch.seq_lens, q_start, q_len, max_q, layer.scaling, sink,
+                                 form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")), n_splits=n_splits)
+        if kt:
+            kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
+        return o
 
     # ---- decode: RoPE + KV store + attention + split merge in one launch -------------------------
     def fused_decode_waves(self, bs: int, head_dim: int, num_kv_splits: int = 0) -> int:

@@ -106,6 +106,52 @@ class DynTanh(nn.Module):
                             want_out=want_out)
 
 
+class StreamRMSNorm(nn.Module):
+    """RMS norm in front of the sublayers of a pre-norm block whose residual stream is fp32 (csrc/layernorm.hip:
+    semipd_rms_stream; fp32 arithmetic whatever the activation type): x / sqrt(mean(x^2) + eps) * (weight + weight_shift);
+    weight_shift 1 is a weight stored around zero.  `seam` is the joint between two sublayers: stream += y, and what the
+    next sublayer reads, next_norm(stream), comes back in the activation type from the same launch."""
+
+    def __init__(self, hidden_size: int, eps: float, weight_shift: float = 0.0, dtype=None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.zeros(hidden_size, dtype=dtype) + (1.0 - weight_shift), requires_grad=False)
+        self.eps, self.weight_shift = float(eps), float(weight_shift)
+
+    def read_stream(self, stream: torch.Tensor) -> torch.Tensor:
+        """self(stream) in the activation type; the stream is left as it is."""
+        return ops.rms_stream(None, stream, self.weight, self.eps, self.weight_shift)
+
+    @staticmethod
+    def seam(y: torch.Tensor, stream: torch.Tensor, next_norm: Optional["StreamRMSNorm"]) -> Optional[torch.Tensor]:
+        """stream += y; returns next_norm(stream) in the activation type (None without next_norm)."""
+        if next_norm is None:
+            return ops.rms_stream(y, stream, None, 0.0, want_out=False)
+        return ops.rms_stream(y, stream, next_norm.weight, next_norm.eps, next_norm.weight_shift)
+
+
+class BigramEmbedding(nn.Module):
+    """Token embedding times a scale plus a row of a hashed table of token pairs, row (previous token * mul_prev + token *
+    mul_cur) mod buckets, the table's last row for the first token of a sequence; the result is the start of an fp32 residual
+    stream.  The previous token of a request is part of its state: an int32 column of the recurrent-state rows, read for the
+    first row of a request's portion and left behind by its last (csrc/layernorm.hip: semipd_embed_bigram)."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, buckets: int, mul_prev: int, mul_cur: int, scale: float,
+                 params_dtype=None):
+        super().__init__()
+        self.buckets, self.mul_prev, self.mul_cur, self.scale = int(buckets), int(mul_prev), int(mul_cur), float(scale)
+        self.weight = nn.Parameter(torch.empty(num_embeddings, embedding_dim, dtype=params_dtype), requires_grad=False)
+        self.bigram = nn.Parameter(torch.empty(self.buckets + 1, embedding_dim, dtype=params_dtype), requires_grad=False)
+
+    def forward(self, input_ids: torch.Tensor, prev_token: torch.Tensor, forward_batch) -> torch.Tensor:
+        """prev_token: the state pool's column for the previous token, viewed as int32 [slots, 1]."""
+        if forward_batch.forward_mode.is_decode():
+            q_start = q_len = None
+        else:
+            q_start, q_len = forward_batch.extend_start_loc, forward_batch.extend_seq_lens
+        return ops.embed_bigram(input_ids, self.weight, self.bigram, self.scale, self.mul_prev, self.mul_cur, self.buckets,
+                                prev_token, forward_batch.state_indices, forward_batch.seq_lens, q_start, q_len)
+
+
 class SiluAndMul(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.silu_and_mul(x)
@@ -664,6 +710,9 @@ class LogitsProcessor(nn.Module):
         self.vocab_size = vocab_size
         self.final_logit_softcapping = final_logit_softcapping
         self.logit_scale = float(logit_scale)     # the fp32 logits are multiplied by it (1: as they are)
+        # soft-capped logits of small batches from the fused head's fp32 logits (models whose cap belongs to the design set
+        # it; the reference's models keep the activation-type matmul in front of the cap, logits_processor.py:394-445)
+        self.softcap_fused = False
 
     def forward(self, input_ids, hidden_states: torch.Tensor, lm_head: VocabParallelEmbedding,
                 forward_batch) -> LogitsProcessorOutput:
@@ -679,11 +728,17 @@ class LogitsProcessor(nn.Module):
         # The fused lm_head + argmax kernel walks the weights once per 64 rows: at 256 rows it takes 1.18 ms where the
         # library GEMM + argmax takes 0.36 (profiles/r02_kbench_all_final_tree.txt), at <= 64 rows it is at par or ahead
         # and returns fp32 logits.  Above that the reference's own form: bf16 GEMM, then fp32 (logits_processor.py:394-445).
-        if get_tensor_model_parallel_world_size() == 1 and self.final_logit_softcapping is None \
+        if get_tensor_model_parallel_world_size() == 1 and (self.final_logit_softcapping is None or self.softcap_fused) \
                 and pruned.shape[0] <= LM_HEAD_FUSED_MAX_ROWS and pruned.dtype in (torch.bfloat16, torch.float16):
             # rows >= vocab_size are padding (vocab_parallel_embedding.py pads to a multiple of 64)
             logits, ids = ops.lm_head_argmax(pruned.contiguous(), lm_head.weight[: self.vocab_size],
                                              return_logits=True)
+            if self.final_logit_softcapping:
+                # cap * tanh(. / cap) on the fp32 logits; it is increasing, so the argmax stands
+                cap = self.final_logit_softcapping
+                logits = cap * torch.tanh(logits * (1.0 / cap)) if self.logit_scale == 1.0 else \
+                    cap * torch.tanh(logits * (self.logit_scale / cap))
+                return LogitsProcessorOutput(logits, next_token_ids=ids if self.logit_scale > 0 else None)
             if self.logit_scale != 1.0:
                 # (a positive factor keeps the argmax; anything else leaves it to the sampler)
                 return LogitsProcessorOutput(logits * self.logit_scale, next_token_ids=ids if self.logit_scale > 0 else None)

@@ -464,3 +464,93 @@ class UngatedMoE(nn.Module):
         if self.w_down_cat is not None:
             return side_by_side_experts(hidden_states, self.w_up, self.w_down_cat, topk_weights, topk_ids)
         return fused_experts_ungated(hidden_states, self.w_up, self.w_down, topk_weights, topk_ids, self.activation)
+
+
+# ---- gated experts with clamps and sigmoid routing ---------------------------------------------------------------------------
+def fused_experts_clamped(hidden_states: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_weights: torch.Tensor,
+                          topk_ids: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """Gated experts whose activation is a = min(gate, limit), b = clamp(up, -limit, limit), a * sigmoid(alpha a) * (b + 1), on
+    the grouped GEMMs of fused_experts (bf16 / f16): align -> GEMM(gate | up) -> activation -> GEMM(down) x routing weight ->
+    sum over the token's experts.  hidden [T, K]; w13 [E, 2F, K] (gate rows, then up rows); w2 [E, K, F]; returns [T, K]."""
+    T, K = hidden_states.shape
+    E, F2, _ = w13.shape
+    F = F2 // 2
+    if T == 0:
+        return hidden_states.new_zeros((0, K))
+    topk = topk_ids.shape[1]
+    dev, dt = hidden_states.device, hidden_states.dtype
+    numel = T * topk
+    tall = (numel >= MOE_TALL_MIN_ROWS and numel >= MOE_TALL_MIN_ROWS_PER_EXPERT * E
+            and ops.moe_gemm_tall_is_supported(hidden_states, w13, False) and F % 64 == 0 and K % 16 == 0)
+    small = (MOE_STREAM_DECODE and T <= MOE_STREAM_MAX_TOKENS and ops.moe_stream_gemm_is_supported(hidden_states, w13, False)
+             and F % 128 == 0 and K % 16 == 0)
+    tall_block = ops.MOE_TALL_BLOCK_M
+    if not tall and not small and (numel >= MOE_MID_MIN_ROWS_PER_EXPERT * E and ops.moe_gemm_tall_is_supported(hidden_states, w13, False)
+                                   and F % 64 == 0 and K % 16 == 0):
+        tall, tall_block = True, 128
+    block_m = tall_block if tall else (min(64, 16 * -(-T // 16)) if small else MOE_BLOCK_M)
+    max_sorted = -(-(numel + E * (block_m - 1)) // block_m) * block_m
+    sorted_ids = torch.empty(max_sorted, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((max_sorted + block_m - 1) // block_m, dtype=torch.int32, device=dev)
+    num_post_pad = torch.empty(1, dtype=torch.int32, device=dev)
+    cumsum = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    ops.moe_align_block_size(topk_ids, E, block_m, sorted_ids, expert_ids, num_post_pad, None, cumsum)
+    c1 = torch.empty((numel, F2), dtype=dt, device=dev)
+    c3 = torch.empty((numel, K), dtype=dt, device=dev)
+    wts = topk_weights.reshape(-1)
+    if small:
+        ops.moe_stream_gemm(hidden_states, w13, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, block_m)
+        c2 = ops.clamped_glu(c1, limit, alpha)
+        ops.moe_stream_gemm(c2, w2, c3, wts, sorted_ids, expert_ids, num_post_pad, numel, 1, True, block_m)
+    elif tall:
+        ops.moe_gemm_tall(hidden_states, w13, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, False,
+                          block_m=block_m)
+        c2 = ops.clamped_glu(c1, limit, alpha)
+        ops.moe_gemm_tall(c2, w2, c3, wts, sorted_ids, expert_ids, num_post_pad, numel, 1, True, False, block_m=block_m)
+    else:
+        ops.moe_grouped_gemm(hidden_states, w13, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, block_m)
+        c2 = ops.clamped_glu(c1, limit, alpha)
+        ops.moe_grouped_gemm(c2, w2, c3, wts, sorted_ids, expert_ids, num_post_pad, numel, 1, True, block_m)
+    return ops.moe_sum(c3.view(T, topk, K))
+
+
+class ClampedGatedMoE(nn.Module):
+    """Mixture of gated feed-forward experts with independent sigmoid scores: the top_k largest scores are kept and divided
+    by their sum (+ 1e-20); expert = down(a * sigmoid(alpha a) * (b + 1)), a = min(gate(x), limit), b = clamp(up(x), -limit,
+    limit).  One GPU per replica.  The router weight is kept in fp32 and multiplied in fp32 (its input is the activation-type
+    rows).  fp32 models and widths the top-k sum refuses evaluate every expert on every token through two plain GEMMs
+    (side_by_side_experts' form with this activation)."""
+
+    RENORM_EPS = 1e-20
+
+    def __init__(self, num_experts: int, top_k: int, hidden_size: int, intermediate_size: int, limit: float,
+                 alpha: float = 1.702, params_dtype=None):
+        super().__init__()
+        if not 0 < top_k <= num_experts:
+            raise ValueError(f"ClampedGatedMoE: top {top_k} of {num_experts} experts")
+        self.num_experts, self.top_k, self.limit, self.alpha = num_experts, top_k, float(limit), float(alpha)
+        self.router = nn.Parameter(torch.empty(num_experts, hidden_size, dtype=torch.float32), requires_grad=False)
+        self.w13 = nn.Parameter(torch.empty(num_experts, 2 * intermediate_size, hidden_size, dtype=params_dtype), requires_grad=False)
+        self.w_down = nn.Parameter(torch.empty(num_experts, hidden_size, intermediate_size, dtype=params_dtype), requires_grad=False)
+        self.w_down_cat: Optional[torch.Tensor] = None
+
+    def side_by_side(self) -> bool:
+        return (self.w13.dtype == torch.float32 or self.w13.shape[2] % 8 != 0 or os.environ.get("SEMIPD_MOE_SIDE_BY_SIDE") == "1")
+
+    def post_load_weights(self):
+        if self.side_by_side():
+            E, K, F = self.w_down.shape
+            self.w_down_cat = self.w_down.permute(1, 0, 2).reshape(K, E * F).contiguous()
+
+    def route(self, hidden_states: torch.Tensor):
+        return ops.topk_sigmoid(ops.router_logits(hidden_states, self.router), self.top_k, True, self.RENORM_EPS)
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        topk_weights, topk_ids = self.route(hidden_states)
+        if self.w_down_cat is not None:
+            from semi_pd_amd.layers.basic import dense_linear
+            E, F2, K = self.w13.shape
+            u = dense_linear(hidden_states, self.w13.view(E * F2, K))
+            y = ops.clamped_glu(u, self.limit, self.alpha, groups=E, topk_weights=topk_weights, topk_ids=topk_ids)
+            return dense_linear(y, self.w_down_cat)
+        return fused_experts_clamped(hidden_states, self.w13, self.w_down, topk_weights, topk_ids, self.limit, self.alpha)

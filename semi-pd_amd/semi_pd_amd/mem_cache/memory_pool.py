@@ -166,10 +166,13 @@ class MHATokenToKVPool:
     kv[L, 2, N + page, Hkv, D] of the module docstring.  `head_num` / `head_dim` / `v_head_dim` may also be given per layer
     (lists of layer_num entries) or with values narrower or wider than keys: the rows then live in ONE byte slab, layer
     after layer, keys [N + page, Hkv_l, D_l] in front of values [N + page, Hkv_l, Dv_l], each region starting on a
-    256-byte boundary -- still one allocation and one IPC handle."""
+    256-byte boundary -- still one allocation and one IPC handle.  `values_in_keys`: a layer's values are the first
+    v_head_dim elements of its key rows (latent attention: one row per token holds the latent and the shared rotated key
+    part, and the latent is the value); such a pool has no value regions, its value buffers are views of the key buffers."""
 
     def __init__(self, size: int, page_size: int, dtype: torch.dtype, head_num, head_dim,
-                 layer_num: int, device: str, bypass_create_buffers: bool = False, v_head_dim=None):
+                 layer_num: int, device: str, bypass_create_buffers: bool = False, v_head_dim=None,
+                 values_in_keys: bool = False):
         assert page_size == 1, "Semi-PD runs with token-granular pages (schedule_batch.py:937)"
         self.size, self.page_size, self.dtype = size, page_size, dtype
         self.layer_num, self.device = layer_num, device
@@ -180,8 +183,11 @@ class MHATokenToKVPool:
         self.head_nums, self.head_dims = per_layer(head_num), per_layer(head_dim)
         self.v_head_dims = per_layer(v_head_dim) if v_head_dim is not None else list(self.head_dims)
         assert len(self.head_nums) == len(self.head_dims) == len(self.v_head_dims) == layer_num
+        self.values_in_keys = bool(values_in_keys)
+        if self.values_in_keys and any(h != 1 or dv > d for h, d, dv in zip(self.head_nums, self.head_dims, self.v_head_dims)):
+            raise ValueError("values_in_keys: one key/value head per layer whose values are a prefix of its key rows")
         self.uniform = (len(set(self.head_nums)) == 1 and len(set(self.head_dims)) == 1
-                        and self.v_head_dims == self.head_dims)
+                        and self.v_head_dims == self.head_dims and not self.values_in_keys)
         self.head_num, self.head_dim = self.head_nums[0], self.head_dims[0]
         self.k_buffer: List[torch.Tensor] = []
         self.v_buffer: List[torch.Tensor] = []
@@ -196,7 +202,8 @@ class MHATokenToKVPool:
             k_off = off
             off = -(-(off + rows * h * d * es) // 256) * 256
             v_off = off
-            off = -(-(off + rows * h * dv * es) // 256) * 256
+            if not self.values_in_keys:
+                off = -(-(off + rows * h * dv * es) // 256) * 256
             out.append((k_off, v_off))
         return out, off
 
@@ -213,12 +220,19 @@ class MHATokenToKVPool:
         rows, es = self.size + self.page_size, self.dtype.itemsize
         for (k_off, v_off), h, d, dv in zip(regions, self.head_nums, self.head_dims, self.v_head_dims):
             self.k_buffer.append(self.slab[k_off: k_off + rows * h * d * es].view(self.dtype).view(rows, h, d))
-            self.v_buffer.append(self.slab[v_off: v_off + rows * h * dv * es].view(self.dtype).view(rows, h, dv))
+            if not self.values_in_keys:
+                self.v_buffer.append(self.slab[v_off: v_off + rows * h * dv * es].view(self.dtype).view(rows, h, dv))
+        self.link_value_views()
+
+    def link_value_views(self):
+        """values_in_keys: the value buffers as views of the key buffers (after creating them or mapping them from another process)."""
+        if self.values_in_keys:
+            self.v_buffer = [k[..., :dv] for k, dv in zip(self.k_buffer, self.v_head_dims)]
 
     def get_kv_size_bytes(self):
         rows, es = self.size + self.page_size, self.dtype.itemsize
         k = sum(rows * h * d * es for h, d in zip(self.head_nums, self.head_dims))
-        v = sum(rows * h * d * es for h, d in zip(self.head_nums, self.v_head_dims))
+        v = 0 if self.values_in_keys else sum(rows * h * d * es for h, d in zip(self.head_nums, self.v_head_dims))
         return k, v
 
     def get_key_buffer(self, layer_id: int):

@@ -27,8 +27,9 @@ def _config_classes():
     from semi_pd_amd.models.llama import LlamaConfig
     from semi_pd_amd.models.kudirax import KudiraxConfig
     from semi_pd_amd.models.opt import OPTConfig
+    from semi_pd_amd.models.penozen import PenozenConfig
     from semi_pd_amd.models.tigotar import TigotarConfig
-    return {"Tigotar": TigotarConfig, "LlamaForCausalLM": LlamaConfig, "OPTForCausalLM": OPTConfig,
+    return {"Tigotar": TigotarConfig, "Penozen": PenozenConfig, "LlamaForCausalLM": LlamaConfig, "OPTForCausalLM": OPTConfig,
             "DeepseekV2ForCausalLM": DeepseekV2Config, "DeepseekV3ForCausalLM": DeepseekV2Config,
             "Kudirax": KudiraxConfig}
 
@@ -204,6 +205,81 @@ def _tigotar_items(config, weights):
         raise RuntimeError(f"checkpoint ended with incomplete stacked parameters: {list(st.pending)[:4]}")
 
 
+_PENOZEN_RE = re.compile(r"^l(\d+)\.(mix|mlp|norm1|norm2)(?:\.(.+))?$")
+_PENOZEN_LATENT_IN = {"q": 0, "dkv": 1, "g": 2}
+_PENOZEN_DELTA_IN = {"q": 0, "k": 1, "v": 2, "g": 3, "a": 4, "b": 5}
+_PENOZEN_DELTA_LEAF = {"q.conv": "conv_q", "k.conv": "conv_k", "v.conv": "conv_v", "A_log": "a_log", "dt_bias": "dt_bias",
+                       "norm": "out_norm"}
+
+
+def _penozen_items(config, weights):
+    """Penozen checkpoint names (embed, bigram, l<i>.norm1|norm2, l<i>.mix.q|dkv|dkv.norm|uk|uv|sink|g|o of a latent-attention
+    layer, l<i>.mix.q|k|v[.conv]|b|a|A_log|dt_bias|norm|g|o of a delta layer, l<i>.mlp.router, l<i>.mlp.e<j>.gate|up|down,
+    final.norm, head) -> product parameters: q | dkv | g (q | k | v | g | a | b) stack into the mixer's merged input
+    projection, the up-projections of keys and values are cut by head, every expert's gate and up rows stack into [E, 2F, W]."""
+    st = _Stacker()
+    top = {"embed": "embed.weight", "bigram": "embed.bigram", "head": "head.weight", "final.norm": "final_norm.weight"}
+    for name, t in weights:
+        if name in top:
+            yield top[name], t
+            continue
+        m = _PENOZEN_RE.match(name)
+        if not m or int(m.group(1)) >= len(config.layers):
+            raise KeyError(f"checkpoint tensor {name} has no counterpart in a Penozen model")
+        i, part, leaf = int(m.group(1)), m.group(2), m.group(3)
+        base = f"layers.{i}."
+        lc = config.layers[i]
+        if part in ("norm1", "norm2"):
+            if leaf is not None:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Penozen model")
+            if part == "norm2" and not lc.experts:
+                continue                      # a layer without feed-forward has no second norm to apply
+            yield base + part + ".weight", t
+        elif part == "mix" and lc.kind == "latent_attention":
+            mc = lc.mixer
+            if leaf in _PENOZEN_LATENT_IN:
+                yield from st.add(base + "mix.in_proj.weight", _PENOZEN_LATENT_IN[leaf], 3, t)
+            elif leaf == "o":
+                yield base + "mix.out_proj.weight", t
+            elif leaf == "dkv.norm":
+                yield base + "mix.latent_norm", t
+            elif leaf == "uk":
+                yield base + "mix.w_uk", t.reshape(mc.heads, mc.dim, mc.kv_rank)
+            elif leaf == "uv":
+                yield base + "mix.w_uv", t.reshape(mc.heads, mc.vdim, mc.kv_rank)
+            elif leaf == "sink":
+                yield base + "mix.sink", t
+            else:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a latent-attention layer")
+        elif part == "mix":
+            if leaf in _PENOZEN_DELTA_IN:
+                yield from st.add(base + "mix.in_proj.weight", _PENOZEN_DELTA_IN[leaf], 6, t)
+            elif leaf == "o":
+                yield base + "mix.out_proj.weight", t
+            elif leaf in _PENOZEN_DELTA_LEAF:
+                yield base + "mix." + _PENOZEN_DELTA_LEAF[leaf], t
+            else:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a delta layer")
+        else:
+            if not lc.experts:
+                raise KeyError(f"checkpoint tensor {name}: layer {i} has no feed-forward")
+            if leaf == "router":
+                yield base + "mlp.router", t
+                continue
+            em = re.match(r"^e(\d+)\.(gate|up|down)$", leaf or "")
+            if not em or int(em.group(1)) >= lc.experts:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Penozen model")
+            e, which = int(em.group(1)), em.group(2)
+            if which == "down":
+                yield from st.add(base + "mlp.w_down", e, lc.experts, t, dim=None)
+            else:
+                # (gate rows of expert e, then its up rows; the experts' blocks follow each other)
+                for done_name, full in st.add(base + "mlp.w13", 2 * e + (which == "up"), 2 * lc.experts, t):
+                    yield done_name, full.reshape(lc.experts, 2 * lc.ff, full.shape[1])
+    if st.pending:
+        raise RuntimeError(f"checkpoint ended with incomplete stacked parameters: {list(st.pending)[:4]}")
+
+
 _EXPERT_RE = re.compile(r"^(.*\.mlp\.experts)\.(\d+)\.(gate_proj|up_proj|down_proj)\.(weight|weight_scale_inv)$")
 
 
@@ -215,6 +291,9 @@ def product_items(config, weights: Iterable[Tuple[str, torch.Tensor]]) -> Iterat
         return
     if arch == "Tigotar":
         yield from _tigotar_items(config, weights)
+        return
+    if arch == "Penozen":
+        yield from _penozen_items(config, weights)
         return
     st = _Stacker()
     tie = bool(getattr(config, "tie_word_embeddings", False))
