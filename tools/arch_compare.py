@@ -1,6 +1,8 @@
 """`python bench.py --arch-compare`: Kudirax next to the Llama-family model of equal size (random weights, one GPU);
 with `--arch-design tigotar`: Tigotar next to Kudirax, the closest model of the framework (fp32 stream, norms on the
-sublayers' outputs, attention over a bounded range of keys through the same kernel family), at equal layer sizes.
+sublayers' outputs, attention over a bounded range of keys through the same kernel family), at equal layer sizes;
+with `--arch-design penozen`: Penozen next to Tigotar (fp32 stream, attention and a recurrence over pooled state rows,
+a mixture of experts behind them).
 
 Two parts, printed as one JSON object:
   * "models": prefill and decode throughput of a few-layer model of each design at layer sizes of real models, both driven
@@ -356,9 +358,220 @@ def main_tigotar(args) -> dict:
     return result
 
 
+PENOZEN_SIZES = {
+    # latent attention: `heads` queries of [dim unrotated | rot rotated] over rows [rank | rot]; delta rule: `heads` value heads of
+    # vdim over `kv` query/key heads of `kdim`; experts as in TIGOTAR_SIZES; two layers of each mixer, in turn
+    "8b-layer": dict(hidden=4096, heads=32, dim=64, rot=64, vdim=128, rank=192, dheads=32, kv=8, kdim=128, dvdim=128, ff=14336,
+                     experts=8, top=2, vocab=32000),
+    "3b-layer": dict(hidden=3072, heads=24, dim=64, rot=64, vdim=128, rank=192, dheads=24, kv=8, kdim=128, dvdim=128, ff=8192,
+                     experts=8, top=2, vocab=32000),
+    "1b-layer": dict(hidden=2048, heads=32, dim=32, rot=32, vdim=64, rank=96, dheads=32, kv=8, kdim=64, dvdim=64, ff=8192,
+                     experts=16, top=4, vocab=32000),
+}
+VALU = 157.3e12      # fp32 vector rate: what a recurrence that is a chain of small matrix-vector steps runs on
+
+
+def _penozen_kernel_pairs(s, t, window, keep, dev):
+    """[(what, Penozen kernel's record, like kernel's record)]: `s` Penozen's layer shape, `t` Tigotar's at the same size."""
+    from semi_pd_amd import ops
+    from semi_pd_amd.layers.moe import fused_experts_clamped, fused_experts_ungated
+    dt = torch.bfloat16
+    W = s["hidden"]
+    H, D, Pr, E, R = s["heads"], s["dim"], s["rot"], s["vdim"], s["rank"]
+    tH, tG, tD = t["heads"], t["kv"], t["dim"]
+    X, K, F = s["experts"], s["top"], s["ff"] // s["top"]
+    out = []
+
+    def rec(tm, nbytes=0.0, flops=0.0, vflops=0.0):
+        frac = max(nbytes / tm / HBM, flops / tm / MFMA, vflops / tm / VALU)
+        return {"us": round(tm * 1e6, 1), "TB_per_s": round(nbytes / tm / 1e12, 2),
+                "TFLOP_per_s": round(max(flops, vflops) / tm / 1e12, 1), "of_roofline": round(frac, 3)}
+
+    # ---- prompt attention: 4 requests x 2048 new tokens ------------------------------------------------------------------
+    B, L = 4, 2048
+    T = B * L
+    pool = torch.randn(T + 1, R + Pr, device=dev, dtype=dt)
+    r2t = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(B, L).contiguous()
+    q = torch.randn(T, H * (R + Pr), device=dev, dtype=dt)
+    o = torch.empty(T, H * R, device=dev, dtype=dt)
+    sink = torch.zeros(H, device=dev)
+    rows = torch.arange(B, device=dev)
+    lens = torch.full((B,), L, device=dev, dtype=torch.int64)
+    q_start = (torch.arange(B, device=dev, dtype=torch.int32) * L)
+    q_len = torch.full((B,), L, device=dev, dtype=torch.int32)
+    # a prompt batch expands keys and values of all heads from the latent rows and attends head by head (the model's path for
+    # batches from 256 new tokens up); the same batch over the latent rows themselves (the path of short portions) for reference
+    from semi_pd_amd.layers.basic import dense_linear
+    w_key = torch.randn(H * (D + Pr), R + Pr, device=dev, dtype=dt) * 0.05
+    w_val = torch.randn(H * E, R + Pr, device=dev, dtype=dt) * 0.05
+    slots = torch.arange(1, T + 1, device=dev)
+    tab = torch.arange(T, device=dev, dtype=torch.int32).view(B, L).contiguous()
+    qh = torch.randn(T, H * (D + Pr), device=dev, dtype=dt)
+    oh = torch.empty(T, H * E, device=dev, dtype=dt)
+    gate = torch.randn(T, H * E, device=dev, dtype=dt)
+
+    def expanded():
+        ctx = ops.gather_rows(pool, slots)
+        keys, vals = dense_linear(ctx, w_key), dense_linear(ctx, w_val)
+        ops.local_attention_fwd(qh, oh, keys.view(-1, H, D + Pr), vals.view(-1, H, E), tab, rows, lens, q_start, q_len, L, 0.1, 0.0, 0,
+                                sink, gate)
+
+    t_new = _timed(expanded)
+    t_lat = _timed(lambda: ops.latent_attention_fwd(q, o, pool, R, r2t, rows, lens, q_start, q_len, L, 0.1, sink))
+    pairs_new = B * L * (L + 1) / 2
+    kp = torch.randn(T + 1, tG, tD, device=dev, dtype=dt)
+    vp = torch.randn(T + 1, tG, tD, device=dev, dtype=dt)
+    tq = torch.randn(T, tH * tD, device=dev, dtype=dt)
+    to = torch.empty(T, tH * tD, device=dev, dtype=dt)
+    hb = torch.full((tH,), -3.0, device=dev)
+    t_old = _timed(lambda: ops.window_attention_fwd(tq, to, kp, vp, r2t, rows, lens, q_start, q_len, L, tD ** -0.5, window, keep, hb,
+                                                    True, None, 1.2))
+    pairs_old = B * sum(min(p + 1, window) + max(0, min(keep, p + 1 - window)) for p in range(L))
+    out.append((f"prompt attention, {B} x {L} tokens ({H} heads of {D} + {Pr} / {E} expanded from latent rows of {R} + {Pr}: gather, two "
+                f"GEMMs, causal softmax with a sink and the output gate; like: window {window} + {keep} kept, sigmoid weights, {tH} heads "
+                f"of {tD})",
+                rec(t_new, flops=2.0 * H * (D + Pr + E) * pairs_new + 2.0 * T * (R + Pr) * H * (D + Pr + E)),
+                rec(t_old, flops=2.0 * tH * 2 * tD * pairs_old)))
+    out.append((f"the same batch over the latent rows themselves ({H} heads x [{R} + {Pr}] queries, one shared key/value row per token: the "
+                "path of portions below 256 tokens; like: the same kernel as above)",
+                rec(t_lat, flops=2.0 * H * (2 * R + Pr) * pairs_new), rec(t_old, flops=2.0 * tH * 2 * tD * pairs_old)))
+    # ---- decode attention: 32 requests at 2000 tokens --------------------------------------------------------------------
+    B2, C = 32, 2000
+    pool2 = torch.randn(B2 * C + 1, R + Pr, device=dev, dtype=dt)
+    r2t2 = (torch.arange(B2 * C, device=dev, dtype=torch.int32) + 1).view(B2, C).contiguous()
+    q2 = torch.randn(B2, H * (R + Pr), device=dev, dtype=dt)
+    o2 = torch.empty(B2, H * R, device=dev, dtype=dt)
+    rows2 = torch.arange(B2, device=dev)
+    lens2 = torch.full((B2,), C, device=dev, dtype=torch.int64)
+    splits = max(1, min(16, 512 // (B2 * ((H + 15) // 16)), C // 128))       # HipAttnBackend.forward_latent's rule on 256 CUs
+    t_new = _timed(lambda: ops.latent_attention_fwd(q2, o2, pool2, R, r2t2, rows2, lens2, None, None, 1, 0.1, sink, n_splits=splits))
+    kp2 = torch.randn(B2 * C + 1, tG, tD, device=dev, dtype=dt)
+    vp2 = torch.randn(B2 * C + 1, tG, tD, device=dev, dtype=dt)
+    tq2 = torch.randn(B2, tH * tD, device=dev, dtype=dt)
+    to2 = torch.empty(B2, tH * tD, device=dev, dtype=dt)
+    t_old = _timed(lambda: ops.window_attention_fwd(tq2, to2, kp2, vp2, r2t2, rows2, lens2, None, None, 1, tD ** -0.5, window, keep, hb,
+                                                    True, None, 1.2))
+    keys_old = min(C, window) + max(0, min(keep, C - window))
+    out.append((f"decode attention, {B2} requests at {C} tokens (every latent row once for all {H} heads, {splits} workgroups share a "
+                f"request's keys, + merge; like: {keys_old} visible keys, {tG} key/value heads)",
+                rec(t_new, nbytes=B2 * (R + Pr) * 2.0 * C, flops=2.0 * B2 * H * (2 * R + Pr) * C),
+                rec(t_old, nbytes=B2 * tG * 2 * tD * 2.0 * keys_old)))
+    # ---- the seam between two sublayers ----------------------------------------------------------------------------------
+    for Tn in (8192, 32):
+        y = torch.randn(Tn, W, device=dev, dtype=dt)
+        res = torch.randn(Tn, W, device=dev, dtype=torch.float32)
+        w = torch.ones(W, device=dev, dtype=dt)
+        b = torch.zeros(W, device=dev, dtype=dt)
+        al = torch.tensor(0.5, device=dev, dtype=dt)
+        t_new = _timed(lambda: ops.rms_stream(y, res, w, 1e-5, 1.0))
+        t_old = _timed(lambda: ops.dyn_tanh(y, (w, b, al), residual=res, params_out=(w, b, al)))
+        nb = Tn * W * (2 + 4 + 4 + 2.0)
+        out.append((f"stream += y, next input = RMS norm(stream), {Tn} rows of {W} (like: stream += squash(y), next = squash(stream))",
+                    rec(t_new, nbytes=nb), rec(t_old, nbytes=nb)))
+    # ---- the step between the projection and the attention ---------------------------------------------------------------
+    Tn = 8192
+    p = torch.randn(Tn, H * (D + Pr) + R + Pr + H * E, device=dev, dtype=dt)
+    pool3 = torch.zeros(Tn + 1, R + Pr, device=dev, dtype=dt)
+    q3 = torch.empty(Tn, H * (R + Pr), device=dev, dtype=dt)
+    loc = torch.arange(1, Tn + 1, device=dev)
+    pos = torch.arange(Tn, device=dev)
+    nw = torch.ones(R, device=dev, dtype=dt)
+    freq = 10000.0 ** (-2.0 * torch.arange(Pr // 2, dtype=torch.float32, device=dev) / Pr)
+    t_new = _timed(lambda: ops.latent_prep(p, H, D, Pr, R, H * (D + Pr), nw, 1e-5, pos, freq, Pr, 1.07, pool3, loc, q3))
+    cols = tH * tD + 2 * tG * tD + 3 * W
+    tp = torch.randn(Tn, cols, device=dev, dtype=dt)
+    kp3 = torch.zeros(Tn + 1, tG, tD, device=dev, dtype=dt)
+    vp3 = torch.zeros(Tn + 1, tG, tD, device=dev, dtype=dt)
+    bq, bk, bv = (torch.zeros(n, device=dev, dtype=dt) for n in (tH * tD, tG * tD, tG * tD))
+    inv_freq = 10000.0 ** (-2.0 * torch.arange(tD // 2, dtype=torch.float32, device=dev) / tD)
+    t_old = _timed(lambda: ops.bias_rope_vnorm_kv_store(tp, tH, tG, tD, tD, tH * tD, tH * tD + tG * tD, bq, bk, bv, pos, inv_freq, tD, 1e-6,
+                                                        kp3, vp3, loc))
+    out.append((f"latent norm + rotation of the shared key part and of every head's rotated query part + pool store, {Tn} tokens "
+                "(like: biases, pair rotation of q and k, value norm, KV store)",
+                rec(t_new, nbytes=Tn * 2.0 * (2 * (R + Pr) + 2 * H * Pr)), rec(t_old, nbytes=Tn * 2.0 * (2 * tH * tD + 4 * tG * tD))))
+    # ---- the recurrences: a prompt batch and a decode batch --------------------------------------------------------------
+    DH, G, KD, VD, taps = s["dheads"], s["kv"], s["kdim"], s["dvdim"], 4
+    gd, hv = G * KD, DH * VD
+    width = 2 * gd + 2 * hv + 2 * DH
+    offs = [0, gd, 2 * gd, 2 * gd + hv, 2 * gd + 2 * hv, 2 * gd + 2 * hv + DH]
+    cw = [torch.randn(n, taps, device=dev, dtype=dt) * 0.5 for n in (gd, gd, hv)]
+    a_log, dt_bias = torch.zeros(DH, device=dev) - 1.0, torch.zeros(DH, device=dev)
+    onw = torch.ones(VD, device=dev, dtype=dt)
+    S = torch.zeros(B2 + 1, DH * KD * VD, device=dev)
+    cs = torch.zeros(B2 + 1, (taps - 1) * (2 * gd + hv), device=dev)
+    dp = torch.randn(T, width, device=dev, dtype=dt)
+    st4 = torch.arange(1, B + 1, device=dev)
+    t_new = _timed(lambda: ops.delta_rule(dp, offs, cw[0], cw[1], cw[2], a_log, dt_bias, onw, 1e-5, S, cs, st4, lens, q_start, q_len, DH, G,
+                                          KD, VD), iters=5, warm=1)
+    Rw = W
+    gp = torch.randn(T, 3 * Rw, device=dev, dtype=dt)
+    gstate = torch.zeros(B2 + 1, Rw, device=dev)
+    yb = torch.empty(T, Rw, device=dev, dtype=dt)
+    bb = torch.zeros(Rw, device=dev, dtype=dt)
+    t_old = _timed(lambda: ops.min_gru(gp, 0, Rw, 2 * Rw, Rw, bb, bb, yb, gstate, st4, lens, q_start, q_len, L))
+    out.append((f"gated delta rule over {B} x {L} tokens, {DH} heads of {KD} x {VD} over {G} key heads (convolutions, unit norms, the "
+                f"recurrence, output norm and gate; 8 flop per element of S and token on the vector units; like: minGRU, {Rw} channels, "
+                "one multiply-add per channel and token, bound by its reads)",
+                rec(t_new, nbytes=T * 2.0 * (width + hv), vflops=8.0 * T * DH * KD * VD), rec(t_old, nbytes=T * Rw * 2.0 * (3 + 1))))
+    dpd = torch.randn(B2, width, device=dev, dtype=dt)
+    st32 = torch.arange(1, B2 + 1, device=dev)
+    t_new = _timed(lambda: ops.delta_rule(dpd, offs, cw[0], cw[1], cw[2], a_log, dt_bias, onw, 1e-5, S, cs, st32, lens2, None, None, DH, G,
+                                          KD, VD))
+    gpd = torch.randn(B2, 3 * Rw, device=dev, dtype=dt)
+    yd = torch.empty(B2, Rw, device=dev, dtype=dt)
+    t_old = _timed(lambda: ops.min_gru(gpd, 0, Rw, 2 * Rw, Rw, bb, bb, yd, gstate, st32, lens2, None, None, 1))
+    out.append((f"gated delta rule decode step, {B2} requests (reads and writes {DH * KD * VD * 4 / 1e6:.1f} MB of state per request; "
+                f"like: minGRU decode step, {Rw * 4 / 1e3:.0f} KB per request, launch-bound)",
+                rec(t_new, nbytes=B2 * DH * KD * VD * 4.0 * 2), rec(t_old, nbytes=B2 * Rw * (2.0 * 4 + 8))))
+    # ---- experts: gated with clamps (three matrices per expert) against ungated (two), same sizes -------------------------------
+    w_up = torch.randn(X, F, W, device=dev, dtype=dt) * 0.02
+    w_down = torch.randn(X, W, F, device=dev, dtype=dt) * 0.02
+    w13 = torch.randn(X, 2 * F, W, device=dev, dtype=dt) * 0.02
+    for Tn in (8192, 32):
+        h = torch.randn(Tn, W, device=dev, dtype=dt)
+        tw, ti = ops.topk_sigmoid(torch.randn(Tn, X, device=dev), K, True, 1e-20)
+        t_new = _timed(lambda: fused_experts_clamped(h, w13, w_down, tw, ti, 7.0, 1.702))
+        t_old = _timed(lambda: fused_experts_ungated(h, w_up, w_down, tw, ti))
+        if Tn > 1024:
+            new, old = rec(t_new, flops=2.0 * Tn * K * 3 * W * F), rec(t_old, flops=2.0 * Tn * K * 2 * W * F)
+        else:   # every expert is touched: the call streams all weights once
+            new, old = rec(t_new, nbytes=X * 3.0 * W * F * 2), rec(t_old, nbytes=X * 2.0 * W * F * 2)
+        out.append((f"experts, {Tn} tokens, top {K} of {X} x {F} (gate | up, clamped gated activation, down; like: up, squared ReLU, down)",
+                    new, old))
+    return out
+
+
+def main_penozen(args) -> dict:
+    from semi_pd_amd.models.penozen import penozen_uniform
+    from semi_pd_amd.models.tigotar import tigotar_uniform
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    window, keep = int(getattr(args, "arch_chunk", 1024) or 1024), 4
+    names = [n for n in (getattr(args, "arch_sizes", "") or ",".join(PENOZEN_SIZES)).split(",") if n]
+    result = {"what": "Penozen next to Tigotar at equal layer sizes", "dtype": "bf16", "data": "synthetic", "models": {}, "kernels": {}}
+    for name in names:
+        s, t = PENOZEN_SIZES[name], TIGOTAR_SIZES[name]
+        result["kernels"][name] = [
+            {"kernel": what, "penozen": new, "like": old,
+             "roofline_fraction_ratio": round(new["of_roofline"] / max(old["of_roofline"], 1e-9), 2)}
+            for what, new, old in _penozen_kernel_pairs(s, t, window, keep, dev)]
+        pcfg = penozen_uniform(s["vocab"], s["hidden"], "adad", s["heads"], s["dim"], s["rot"], s["vdim"], s["rank"], s["dheads"], s["kv"],
+                               s["kdim"], s["dvdim"], s["experts"], s["top"], s["ff"] // s["top"])
+        tcfg = tigotar_uniform(t["vocab"], t["hidden"], 4, t["heads"], t["kv"], t["dim"], t["dim"], t["hidden"], t["experts"], t["top"],
+                               t["ff"] // t["top"], window, keep, loop=None)
+        result["models"][name] = {
+            "layers": 4,
+            "penozen": _model_throughput(pcfg, 2048, 4, 32, 1100, 20),
+            "tigotar": _model_throughput(tcfg, 2048, 4, 32, 1100, 20)}
+    print(json.dumps(result), flush=True)
+    return result
+
+
 def main(args) -> dict:
     if getattr(args, "arch_design", "kudirax") == "tigotar":
         return main_tigotar(args)
+    if getattr(args, "arch_design", "kudirax") == "penozen":
+        return main_penozen(args)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     chunk = int(getattr(args, "arch_chunk", 1024) or 0)
