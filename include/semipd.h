@@ -889,14 +889,16 @@ int semipd_embed_bigram(const int64_t* ids, const void* embed, const void* bigra
                         int64_t mul_cur, int64_t buckets, int32_t* prev, int64_t prev_ld, const int64_t* state_indices,
                         const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len, int64_t batch,
                         int64_t num_tokens, float* out, int64_t width, int dtype, void* stream);
-/* Latent attention, the step behind the projection GEMM.  Row t of proj: per head [dim unrotated | rot_dim rotated] query
- * elements from column 0; at column c_off the latent [rank] and one rotated key part [rot_dim].  pool[loc[t]] <-
- * [rms_norm(latent) * norm_weight | key part turned]; q_out[t, h * q_head_stride + q_head_off ...) <- head h's rotated part
- * turned (q_out may be proj itself: in place) (neighbouring pairs of the first rot_dims elements by positions[t] * freq[i], cos and sin times mscale; fp32). */
+/* Latent attention, the step behind the projection GEMMs.  Row t of proj: per head [dim unrotated | rot_dim rotated] query
+ * elements from column 0; row t of latent: the latent [rank] and one rotated key part [rot_dim] (the same rows at another
+ * column, or another projection's).  pool[loc[t]] <- [rms_norm(latent) * norm_weight | key part turned];
+ * q_out[t, h * q_head_stride + q_head_off ...) <- head h's rotated part turned (q_out may be proj itself: in place).  Turned:
+ * pair i of the first rot_dims elements -- (2i, 2i + 1), with `halves` (i, i + rot_dims / 2) -- by positions[t] * freq[i],
+ * cos and sin times mscale; fp32. */
 int semipd_latent_prep(const void* proj, int64_t ld, int64_t num_tokens, int num_heads, int dim, int rot_dim, int rank,
-                       int64_t c_off, const void* norm_weight, float eps, const int64_t* positions, const float* freq,
-                       int rot_dims, float mscale, void* pool, int64_t pool_ld, const int64_t* loc, void* q_out,
-                       int64_t q_ld, int q_head_stride, int q_head_off, int dtype, void* stream);
+                       const void* latent, int64_t latent_ld, int halves, const void* norm_weight, float eps,
+                       const int64_t* positions, const float* freq, int rot_dims, float mscale, void* pool, int64_t pool_ld,
+                       const int64_t* loc, void* q_out, int64_t q_ld, int q_head_stride, int q_head_off, int dtype, void* stream);
 /* Causal softmax attention (+ exp(sink[h]) in the denominator) of num_heads queries [rank + rot_dim] per token over pool
  * rows [rank + rot_dim] found through req_to_token; the value of a row is its first `rank` elements; out [T, heads * rank].
  * Batch description and `form` as in semipd_local_attention.  n_splits > 1 (decode batches on the matrix-core form): that
@@ -935,6 +937,60 @@ int semipd_topk_sigmoid(const void* gating, float* topk_weights, int32_t* topk_i
 /* x [rows, width] (row stride x_ld) <- x * sigmoid(gate), fp32 arithmetic.  No reference counterpart. */
 int semipd_sigmoid_gate(void* x, int64_t x_ld, const void* gate, int64_t gate_ld, int64_t rows, int64_t width, int dtype,
                         void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Norm after the sum on an fp32 stream, token shift, attention whose   */
+/* heads talk, state-space recurrence                                   */
+/* ------------------------------------------------------------------ */
+/* x [rows, heads * head_width] <- x * sigmoid(gate[row, head]), fp32 arithmetic.  No reference counterpart. */
+int semipd_sigmoid_gate_heads(void* x, int64_t x_ld, const void* gate, int64_t gate_ld, int64_t rows, int64_t heads,
+                              int64_t head_width, int dtype, void* stream);
+/* out (fp32 [num_tokens, width]) = embed[ids[t]] * scale. */
+int semipd_embed_stream(const int64_t* ids, const void* embed, float scale, int64_t num_tokens, float* out, int64_t width,
+                        int dtype, void* stream);
+/* stream (fp32 rows, in place) <- rms_norm(alpha * stream + layer_scale * y) * weight (y, layer_scale may be NULL); when out
+ * is given it receives the new stream in `dtype`, or with shift_mu (batches of ONE row per request only) the token-shifted
+ * stream s + (prev - s) * shift_mu, prev the request's row of `prev` (zeros when seq_lens[row] <= 1), which is then
+ * replaced by s.  No reference counterpart. */
+int semipd_postnorm_stream(const void* y, int64_t y_ld, const void* layer_scale, float* stream, int64_t stream_ld, float alpha,
+                           const void* weight, float eps, void* out, int64_t out_ld, const void* shift_mu, float* prev,
+                           int64_t prev_ld, const int64_t* state_indices, const int64_t* seq_lens, int64_t rows, int64_t width,
+                           int dtype, void* stream_handle);
+/* out[t] = s_t + (s_(t-1) - s_t) * mu in `dtype`, s the fp32 stream; the row in front of a request's portion is the request's
+ * row of `prev` (zeros at position 0); the portion's last row is left there.  Batch description as in
+ * semipd_local_attention.  No reference counterpart. */
+int semipd_token_shift(const float* stream, int64_t stream_ld, const void* mu, float* prev, int64_t prev_ld,
+                       const int64_t* state_indices, const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len,
+                       int64_t batch, int64_t num_tokens, void* out, int64_t out_ld, int64_t width, int dtype, void* stream_handle);
+/* Rows of qkv hold q | k | v at columns 0, k_off, v_off.  q and k: RMS norm over the whole projection (all heads at once)
+ * times q_weight / k_weight (NULL: no norm), the first rot_dims elements of every head turned (pairs as in
+ * semipd_latent_prep), query head h times head_scale[h] (NULL: 1); q in place, k / v into the pools at loc. */
+int semipd_qk_norm_rope_kv_store(void* qkv, int64_t ld, int64_t num_tokens, int num_q_heads, int num_kv_heads, int qk_dim,
+                                 int v_dim, int64_t k_off, int64_t v_off, const void* q_weight, const void* k_weight, float eps,
+                                 const int64_t* positions, const float* freq, int rot_dims, int halves, float mscale,
+                                 const float* head_scale, void* k_pool, void* v_pool, const int64_t* loc, int dtype, void* stream);
+/* semipd_local_attention (causal, softmax) whose value row of a slot is ONE head of v_row elements read by the queries of
+ * every key/value head: out [T, heads * v_row]. */
+int semipd_shared_value_attention(const void* q, int64_t q_ld, void* out, int64_t out_ld, const void* k_pool, const void* v_pool,
+                                  const int32_t* req_to_token, int64_t req_to_token_stride, const int64_t* req_pool_indices,
+                                  const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len, int64_t batch,
+                                  int64_t num_tokens, int64_t max_q_len, int num_q_heads, int num_kv_heads, int qk_dim, int v_row,
+                                  float scale, int form, int dtype, void* stream);
+/* out[t, h, :] = sum_g talk[h, g] * parts[t, g, c(h), :], parts [T, heads, kv heads, v_dim], c(h) the key/value head of h. */
+int semipd_talk_mix(const void* parts, int64_t parts_ld, const float* talk, void* out, int64_t out_ld, int64_t num_tokens,
+                    int num_q_heads, int num_kv_heads, int v_dim, int dtype, void* stream);
+/* fp32 elements of a work row of semipd_state_space. */
+int64_t semipd_state_space_work_width(int num_heads, int groups, int state, int v_dim);
+/* The state-space recurrence behind its projection GEMM: rows [z | x | B | C | dt] at z_off, x_off (x | B | C, the
+ * convolution's channels), dt_off; conv_w [C, taps], conv_b [C] (may be NULL); dt_bias, a_log, d_skip fp32 [H]; norm_w
+ * [H * v_dim]; state fp32 [slots, H * state * v_dim] and conv_state fp32 [slots, (taps - 1) * C] are column ranges of the
+ * requests' state rows; out [T, H * v_dim].  fused_decode: batches of one row per request take one launch. */
+int semipd_state_space(const void* proj, int64_t ld, int64_t z_off, int64_t x_off, int64_t dt_off, const void* conv_w,
+                       const void* conv_b, const float* dt_bias, const float* a_log, const float* d_skip, const void* norm_w,
+                       int norm_groups, float eps, float* work, int64_t work_ld, float* state, int64_t state_ld, float* conv_state,
+                       int64_t conv_ld, const int64_t* state_indices, const int64_t* seq_lens, const int32_t* q_start,
+                       const int32_t* q_len, int64_t batch, int64_t num_tokens, int num_heads, int groups, int state_size, int v_dim,
+                       int taps, void* out, int64_t out_ld, int fused_decode, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

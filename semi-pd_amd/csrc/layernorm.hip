@@ -405,6 +405,119 @@ __global__ void __launch_bounds__(256) sigmoid_gate_kernel(T* __restrict__ x, in
   }
 }
 
+// ---- x <- x * sigmoid(gate[head]): one gate per (row, head) over the head's `head_width` elements, fp32 arithmetic
+template <typename T>
+__global__ void __launch_bounds__(256) sigmoid_gate_heads_kernel(T* __restrict__ x, int64_t x_ld, const T* __restrict__ gate,
+                                                                 int64_t gate_ld, int64_t rows, int64_t heads, int64_t head_width) {
+  const int64_t width = heads * head_width, n = rows * width;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / width, c = i - r * width;
+    const float g = Elem<T>::to_f(gate[r * gate_ld + c / head_width]);
+    x[r * x_ld + c] = Elem<T>::from_f(Elem<T>::to_f(x[r * x_ld + c]) / (1.0f + expf(-g)));
+  }
+}
+
+// ---- token embedding times a scale as the start of an fp32 stream
+template <typename T>
+__global__ void __launch_bounds__(256) embed_stream_kernel(const int64_t* __restrict__ ids, const T* __restrict__ embed, float scale,
+                                                           float* __restrict__ out, int64_t width) {
+  const int64_t t = blockIdx.x;
+  const T* e = embed + ids[t] * width;
+  for (int64_t i = threadIdx.x; i < width; i += 256) out[t * width + i] = Elem<T>::to_f(e[i]) * scale;
+}
+
+// The request that owns row t of a batch, the row's index in the request's portion, the portion's length and the position
+// of its first row (q_start == NULL: row t is request t's newest token).
+__device__ __forceinline__ bool portion_of_row(int64_t t, int64_t batch, const int64_t* seq_lens, const int32_t* q_start,
+                                               const int32_t* q_len, int& b, int64_t& li, int64_t& n, int64_t& first_pos) {
+  if (q_start == nullptr) {
+    b = (int)t; li = 0; n = 1; first_pos = seq_lens[b] - 1;
+    return first_pos >= 0;
+  }
+  for (int r = 0; r < (int)batch; ++r) {
+    const int64_t s = q_start[r], m = q_len[r];
+    if (t >= s && t < s + m) {
+      b = r; li = t - s; n = m; first_pos = seq_lens[r] - m;
+      return true;
+    }
+  }
+  return false;
+}
+
+// ---- norm AFTER the sum on an fp32 stream, with a per-channel scale on the sublayer's result:
+//     stream <- (alpha stream + ls * y) / sqrt(mean((alpha stream + ls * y)^2) + eps) * weight          (fp32, in place)
+// and, when `out` is given, what the next sublayer reads, in the activation type: the new stream itself, or -- with `mu` --
+// the token-shifted stream  s + (s_prev - s) * mu,  s_prev the previous token's new stream.  The shifted form is for
+// batches of ONE row per request (q_start == NULL): s_prev is the request's entry of `prev` (zeros at position 0), which
+// the row then replaces by its own stream.  A workgroup per row.
+template <typename T>
+__global__ void __launch_bounds__(256) postnorm_stream_kernel(const T* __restrict__ y, int64_t y_ld, const T* __restrict__ ls,
+                                                              float* __restrict__ stream, int64_t s_ld, float alpha,
+                                                              const T* __restrict__ w, float eps, T* __restrict__ out, int64_t out_ld,
+                                                              const T* __restrict__ mu, float* __restrict__ prev, int64_t prev_ld,
+                                                              const int64_t* __restrict__ state_indices,
+                                                              const int64_t* __restrict__ seq_lens, int64_t width) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  float* x = stream + r * s_ld;
+  float q = 0.f;
+  for (int64_t i = threadIdx.x; i < width; i += 256) {
+    float v = alpha * x[i];
+    if (y) v += Elem<T>::to_f(y[r * y_ld + i]) * (ls ? Elem<T>::to_f(ls[i]) : 1.0f);
+    x[i] = v;
+    q += v * v;
+  }
+  const float rs = 1.0f / sqrtf(block_sum(q, red) / (float)width + eps);
+  float* pv = nullptr;
+  bool first = true;
+  if (mu) {
+    pv = prev + state_indices[r] * prev_ld;
+    first = seq_lens[r] <= 1;
+  }
+  for (int64_t i = threadIdx.x; i < width; i += 256) {          // (every thread re-reads the elements it wrote itself)
+    const float v = x[i] * rs * Elem<T>::to_f(w[i]);
+    x[i] = v;
+    if (!out) continue;
+    if (mu) {
+      const float before = first ? 0.f : pv[i];
+      pv[i] = v;
+      out[r * out_ld + i] = Elem<T>::from_f(v + (before - v) * Elem<T>::to_f(mu[i]));
+    } else {
+      out[r * out_ld + i] = Elem<T>::from_f(v);
+    }
+  }
+}
+
+// ---- token shift on an fp32 stream: out[t] = s_t + (s_(t-1) - s_t) * mu in the activation type, s_(t-1) the previous row of
+// the request's portion, for the portion's first row the request's entry of `prev` (zeros at position 0).  The workgroup of
+// a portion's first row also leaves the portion's LAST row in `prev`, element by element behind its own read.
+template <typename T>
+__global__ void __launch_bounds__(256) token_shift_kernel(const float* __restrict__ stream, int64_t s_ld, const T* __restrict__ mu,
+                                                          float* __restrict__ prev, int64_t prev_ld,
+                                                          const int64_t* __restrict__ state_indices,
+                                                          const int64_t* __restrict__ seq_lens, const int32_t* __restrict__ q_start,
+                                                          const int32_t* __restrict__ q_len, int64_t batch, T* __restrict__ out,
+                                                          int64_t out_ld, int64_t width) {
+  const int64_t t = blockIdx.x;
+  int b;
+  int64_t li, n, first_pos;
+  if (!portion_of_row(t, batch, seq_lens, q_start, q_len, b, li, n, first_pos)) return;
+  const float* x = stream + t * s_ld;
+  if (li > 0) {
+    const float* xp = stream + (t - 1) * s_ld;
+    for (int64_t i = threadIdx.x; i < width; i += 256)
+      out[t * out_ld + i] = Elem<T>::from_f(x[i] + (xp[i] - x[i]) * Elem<T>::to_f(mu[i]));
+    return;
+  }
+  float* pv = prev + state_indices[b] * prev_ld;
+  const float* last = stream + (t + n - 1) * s_ld;
+  for (int64_t i = threadIdx.x; i < width; i += 256) {
+    const float before = first_pos == 0 ? 0.f : pv[i];
+    pv[i] = last[i];
+    out[t * out_ld + i] = Elem<T>::from_f(x[i] + (before - x[i]) * Elem<T>::to_f(mu[i]));
+  }
+}
+
 }  // namespace semipd
 
 using namespace semipd;
@@ -582,4 +695,62 @@ extern "C" int semipd_sigmoid_gate(void* x, int64_t x_ld, const void* gate, int6
                         hipLaunchKernelGGL((sigmoid_gate_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (T*)x, x_ld,
                                            (const T*)gate, gate_ld, rows, width));
   return launch_status("sigmoid_gate");
+}
+
+
+extern "C" int semipd_sigmoid_gate_heads(void* x, int64_t x_ld, const void* gate, int64_t gate_ld, int64_t rows, int64_t heads,
+                                         int64_t head_width, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(rows >= 0 && heads > 0 && head_width > 0 && x_ld >= heads * head_width && gate_ld >= heads, SEMIPD_EINVAL,
+                   "sigmoid_gate_heads: bad sizes");
+  if (rows == 0) return 0;
+  SEMIPD_CHECK_ARG(x && gate, SEMIPD_EINVAL, "sigmoid_gate_heads: null pointer");
+  const int64_t n = rows * heads * head_width;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((sigmoid_gate_heads_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (T*)x, x_ld,
+                                           (const T*)gate, gate_ld, rows, heads, head_width));
+  return launch_status("sigmoid_gate_heads");
+}
+
+extern "C" int semipd_embed_stream(const int64_t* ids, const void* embed, float scale, int64_t num_tokens, float* out, int64_t width,
+                                   int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && width > 0, SEMIPD_EINVAL, "embed_stream: bad sizes");
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(ids && embed && out, SEMIPD_EINVAL, "embed_stream: null pointer");
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((embed_stream_kernel<T>), dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream), ids,
+                                           (const T*)embed, scale, out, width));
+  return launch_status("embed_stream");
+}
+
+extern "C" int semipd_postnorm_stream(const void* y, int64_t y_ld, const void* layer_scale, float* stream, int64_t stream_ld,
+                                      float alpha, const void* weight, float eps, void* out, int64_t out_ld, const void* shift_mu,
+                                      float* prev, int64_t prev_ld, const int64_t* state_indices, const int64_t* seq_lens,
+                                      int64_t rows, int64_t width, int dtype, void* stream_handle) {
+  SEMIPD_CHECK_ARG(rows >= 0 && width > 0, SEMIPD_EINVAL, "postnorm_stream: bad sizes");
+  if (rows == 0) return 0;
+  SEMIPD_CHECK_ARG(stream && weight, SEMIPD_EINVAL, "postnorm_stream: null pointer");
+  SEMIPD_CHECK_ARG(shift_mu == nullptr || (out && prev && state_indices && seq_lens && prev_ld >= width), SEMIPD_EINVAL,
+                   "postnorm_stream: the shifted form needs out, the previous rows and the batch's state rows and lengths");
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((postnorm_stream_kernel<T>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream_handle),
+                                           (const T*)y, y_ld, (const T*)layer_scale, stream, stream_ld, alpha, (const T*)weight, eps,
+                                           (T*)out, out_ld, (const T*)shift_mu, prev, prev_ld, state_indices, seq_lens, width));
+  return launch_status("postnorm_stream");
+}
+
+extern "C" int semipd_token_shift(const float* stream, int64_t stream_ld, const void* mu, float* prev, int64_t prev_ld,
+                                  const int64_t* state_indices, const int64_t* seq_lens, const int32_t* q_start,
+                                  const int32_t* q_len, int64_t batch, int64_t num_tokens, void* out, int64_t out_ld, int64_t width,
+                                  int dtype, void* stream_handle) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && batch >= 0 && width > 0 && prev_ld >= width, SEMIPD_EINVAL, "token_shift: bad sizes");
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(stream && mu && prev && state_indices && seq_lens && out, SEMIPD_EINVAL, "token_shift: null pointer");
+  SEMIPD_CHECK_ARG((q_start == nullptr) == (q_len == nullptr) && (q_start != nullptr || num_tokens == batch), SEMIPD_EINVAL,
+                   "token_shift: q_start and q_len come together; without them one row per request");
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((token_shift_kernel<T>), dim3((unsigned)num_tokens), dim3(256), 0,
+                                           as_stream(stream_handle), stream, stream_ld, (const T*)mu, prev, prev_ld, state_indices,
+                                           seq_lens, q_start, q_len, batch, (T*)out, out_ld, width));
+  return launch_status("token_shift");
 }

@@ -279,8 +279,10 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_vec_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------ latent attention: preparation
-// Rows of `proj` hold, per head, [D unrotated | P rotated] query elements from column 0 and, at column c_off, the latent
-// [R] and one rotated key part [P] shared by all heads.  One workgroup per token:
+// Rows of `proj` hold, per head, [D unrotated | P rotated] query elements from column 0; rows of `latent` (the same rows at
+// another column, or the rows of another projection) the latent [R] and one rotated key part [P] shared by all heads.
+// `halves`: pair i of a rotation is elements (i, i + rot_dims / 2) instead of the neighbours (2i, 2i + 1).
+// One workgroup per token:
 //   latent / sqrt(mean(latent^2) + eps) * weight -> pool row [0, R); the key part, its first rot_dims elements turned
 //   in neighbouring pairs by position * freq[i] (cos and sin times `mscale`) -> pool row [R, R + P);
 //   the rotated part of every head's query, turned the same way -> q_out[t, h * q_head_stride + q_head_off ...): behind
@@ -288,7 +290,8 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_vec_kernel(
 // Angles, the norm and the products are fp32; one rounding on the way out.
 template <typename T>
 __global__ void __launch_bounds__(256) latent_prep_kernel(const T* __restrict__ proj, int64_t ld, int64_t num_tokens, int H, int D,
-                                                          int P, int R, int64_t c_off, const T* __restrict__ norm_w, float eps,
+                                                          int P, int R, const T* __restrict__ latent, int64_t latent_ld,
+                                                          int halves, const T* __restrict__ norm_w, float eps,
                                                           const int64_t* __restrict__ positions, const float* __restrict__ freq,
                                                           int rot_dims, float mscale, T* __restrict__ pool, int64_t pool_ld,
                                                           const int64_t* __restrict__ loc, T* __restrict__ q_out, int64_t q_ld,
@@ -301,7 +304,7 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(const T* __restrict__ 
   const int64_t t = blockIdx.x;
   const float pos = (float)positions[t];
   const int half = rot_dims >> 1;
-  const T* c = proj + t * ld + c_off;
+  const T* c = latent + t * latent_ld;
   T* row = pool + loc[t] * pool_ld;
   if (wave == 0) {
     float sq = 0.f;
@@ -330,12 +333,103 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(const T* __restrict__ 
     T* dst = u == 0 ? row + R : q_out + t * q_ld + (int64_t)(u - 1) * q_head_stride + q_head_off;
     if (i < half) {
       const float cs = cs_l[2 * i], sn = cs_l[2 * i + 1];
-      const float x1 = Elem<T>::to_f(src[2 * i]), x2 = Elem<T>::to_f(src[2 * i + 1]);
-      dst[2 * i] = Elem<T>::from_f(x1 * cs - x2 * sn);
-      dst[2 * i + 1] = Elem<T>::from_f(x2 * cs + x1 * sn);
+      const int i1 = halves ? i : 2 * i, i2 = halves ? i + half : 2 * i + 1;     // pair i: (i, i + dims / 2) or (2i, 2i + 1)
+      const float x1 = Elem<T>::to_f(src[i1]), x2 = Elem<T>::to_f(src[i2]);
+      dst[i1] = Elem<T>::from_f(x1 * cs - x2 * sn);
+      dst[i2] = Elem<T>::from_f(x2 * cs + x1 * sn);
     } else {
       dst[rot_dims + (i - half)] = src[rot_dims + (i - half)];
     }
+  }
+}
+
+
+// ------------------------------------------------------------------------------------------------ attention whose heads talk
+// Preparation behind the q | k | v projection of a layer whose queries and keys are normed over the WHOLE projection (all
+// heads at once): q / sqrt(mean(q^2) + eps) * q_weight over its H * D elements, the same for k over G * D, then the first
+// rot_dims elements of every head turned by position * freq[i] (pair i = elements (2i, 2i + 1), or (i, i + rot_dims / 2)
+// with `halves`; cos and sin times `mscale`), then every query head times head_scale[h] (a per-head temperature, folded into the query in fp32).
+// q in place, k and v into the pools at loc.  A workgroup per token; norms, angles and products fp32, one rounding.
+template <typename T>
+__global__ void __launch_bounds__(256) qk_norm_rope_kv_store_kernel(T* __restrict__ qkv, int64_t ld, int H, int G, int D, int E,
+                                                                    int64_t k_off, int64_t v_off, const T* __restrict__ q_w,
+                                                                    const T* __restrict__ k_w, float eps,
+                                                                    const int64_t* __restrict__ positions,
+                                                                    const float* __restrict__ freq, int rot_dims, int halves,
+                                                                    float mscale, const float* __restrict__ head_scale,
+                                                                    T* __restrict__ k_pool,
+                                                                    T* __restrict__ v_pool, const int64_t* __restrict__ loc) {
+  extern __shared__ float cs_l[];          // [rot_dims / 2][2]
+  __shared__ float red[16];
+  const int tid = threadIdx.x;
+  const int64_t t = blockIdx.x;
+  T* row = qkv + t * ld;
+  const int64_t slot = loc[t];
+  const float pos = (float)positions[t];
+  const int half = rot_dims >> 1;
+  for (int i = tid; i < half; i += 256) {
+    float sn, cs;
+    sincosf(pos * freq[i], &sn, &cs);
+    cs_l[2 * i] = cs * mscale;
+    cs_l[2 * i + 1] = sn * mscale;
+  }
+  float sq = 0.f, sk = 0.f;
+  if (q_w)
+    for (int i = tid; i < H * D; i += 256) {
+      const float v = Elem<T>::to_f(row[i]);
+      sq += v * v;
+    }
+  if (k_w)
+    for (int i = tid; i < G * D; i += 256) {
+      const float v = Elem<T>::to_f(row[k_off + i]);
+      sk += v * v;
+    }
+  sq = block_sum(sq, red);
+  sk = block_sum(sk, red);                 // (block_sum's first barrier also orders the reads of red above and cs_l's writes)
+  const float rq = q_w ? 1.0f / sqrtf(sq / (float)(H * D) + eps) : 1.0f;
+  const float rk = k_w ? 1.0f / sqrtf(sk / (float)(G * D) + eps) : 1.0f;
+  __syncthreads();
+  const int per = half + (D - rot_dims);             // items of a head: the pairs, then the elements that pass unchanged
+  for (int item = tid; item < (H + G) * per; item += 256) {
+    const int u = item / per, i = item % per;
+    const bool is_q = u < H;
+    const int h = is_q ? u : u - H;
+    const T* src = is_q ? row + (int64_t)h * D : row + k_off + (int64_t)h * D;
+    const T* wv = is_q ? (q_w ? q_w + (int64_t)h * D : nullptr) : (k_w ? k_w + (int64_t)h * D : nullptr);
+    T* dst = is_q ? row + (int64_t)h * D : k_pool + (slot * G + h) * D;
+    const float r = is_q ? rq : rk;
+    const float hs = (is_q && head_scale) ? head_scale[h] : 1.0f;
+    if (i < half) {
+      const int i1 = halves ? i : 2 * i, i2 = halves ? i + half : 2 * i + 1;
+      const float cs = cs_l[2 * i], sn = cs_l[2 * i + 1];
+      const float x1 = Elem<T>::to_f(src[i1]) * r * (wv ? Elem<T>::to_f(wv[i1]) : 1.0f);
+      const float x2 = Elem<T>::to_f(src[i2]) * r * (wv ? Elem<T>::to_f(wv[i2]) : 1.0f);
+      dst[i1] = Elem<T>::from_f((x1 * cs - x2 * sn) * hs);
+      dst[i2] = Elem<T>::from_f((x2 * cs + x1 * sn) * hs);
+    } else {
+      const int e = rot_dims + (i - half);
+      dst[e] = Elem<T>::from_f(Elem<T>::to_f(src[e]) * r * (wv ? Elem<T>::to_f(wv[e]) : 1.0f) * hs);
+    }
+  }
+  for (int i = tid; i < G * E; i += 256) v_pool[slot * (int64_t)G * E + i] = row[v_off + i];
+}
+
+// The heads' attention weights mixed AFTER the softmax: w'_h(i, j) = sum_g talk[h, g] w_g(i, j), and head h applies w'_h to
+// the values of its own key/value head c(h).  The sum over the keys is linear, so
+//     out_h = sum_g talk[h, g] * (w_g applied to the values of head c(h)),
+// and `parts` [T, H, G, E] holds w_g applied to the values of EVERY key/value head (attention whose value row is shared).
+// A workgroup per token, a thread per element of out [T, H * E]; fp32 sums.
+template <typename T>
+__global__ void __launch_bounds__(256) talk_mix_kernel(const T* __restrict__ parts, int64_t p_ld, const float* __restrict__ talk,
+                                                       T* __restrict__ out, int64_t out_ld, int H, int G, int E) {
+  const int64_t t = blockIdx.x;
+  const T* p = parts + t * p_ld;
+  const int per = H / G;
+  for (int i = threadIdx.x; i < H * E; i += 256) {
+    const int h = i / E, e = i - h * E, c = h / per;
+    float y = 0.f;
+    for (int g = 0; g < H; ++g) y += talk[h * H + g] * Elem<T>::to_f(p[((int64_t)g * G + c) * E + e]);
+    out[t * out_ld + i] = Elem<T>::from_f(y);
   }
 }
 
@@ -361,6 +455,7 @@ struct LocalAttnArgs {
   int64_t k_ld, v_ld;              // elements between the rows of two slots (G * D and G * E for pools of their own)
   int n_splits;                    // decode form: workgroups that share the keys of one (request, kv head, 16 q heads) (0 / 1: one)
   float* partial;                  // [rows, H, n_splits, E + 2] fp32: unnormalised sums, running maximum, denominator
+  int v_shared;                    // 1: the value row of a slot is ONE head of E elements that every key/value head's queries read
 };
 
 // first visible position of the contiguous range that ends at the query (the kept first positions come on top)
@@ -461,7 +556,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
       for (int jj = 0; jj < n; ++jj) {
         const float pj = __shfl(p, jj, 64);
         const int sj = __shfl(slot, jj, 64);
-        const T* v = vp + (int64_t)sj * a.v_ld + (int64_t)g * E;
+        const T* v = vp + (int64_t)sj * a.v_ld + (a.v_shared ? 0 : (int64_t)g * E);
 #pragma unroll
         for (int u = 0; u < NA; ++u) {
           const int e = lane + 64 * u;
@@ -802,11 +897,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
   const int64_t n_first = keep < blk_lo ? keep : blk_lo;
   if (n_first > 0)
     key_walk<T, ND, NE, 256, true, SIG>(
-        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (a.v_shared ? 0 : (int64_t)gk * E),
         a.v_ld, row, 0, n_first - 1, 32, v_lds, tid, a.scale, a.cap, [&](int64_t j) { return q_ok && j < n_first; },
         [&](int64_t) { return wave_on; }, r, g, nullptr, 0, hb);
   key_walk<T, ND, NE, 256, true, SIG>(
-      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (a.v_shared ? 0 : (int64_t)gk * E),
       a.v_ld, row, blk_lo, blk_hi, 32, v_lds, tid, a.scale, a.cap,
       [&](int64_t j) { return q_ok && j <= my_pos && (j >= my_lo || j < keep); },
       [&](int64_t j0) { return wave_on && j0 <= w_hi && (j0 + 31 >= w_lo || j0 < keep); }, r, g, nullptr, blk_lo, hb);
@@ -906,11 +1001,11 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
   // the kept first positions in front of the window (none without one), then the range that ends at the query
   if (n_first > 0)
     key_walk<T, ND, NE, 64, false, SIG>(
-        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (a.v_shared ? 0 : (int64_t)gk * E),
         a.v_ld, row, (int64_t)32 * wave, n_first - 1, 32 * NW, mine_b, lane, a.scale, a.cap,
         [&](int64_t j) { return j < n_first; }, [&](int64_t) { return true; }, r, g, nullptr, 0, hb);
   key_walk<T, ND, NE, 64, false, SIG>(
-      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (int64_t)gk * E,
+      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, a.k_ld, (const T*)a.v_pool + (a.v_shared ? 0 : (int64_t)gk * E),
       a.v_ld, row, lo + 32 * wave, pos, 32 * NW, mine_b, lane, a.scale, a.cap, [&](int64_t j) { return j <= pos; },
       [&](int64_t) { return true; }, r, g, idx_fits ? idx_lds : nullptr, lo, hb);
   float l = st.l;
@@ -1097,7 +1192,7 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
   SEMIPD_CHECK_ARG(batch >= 0 && num_tokens >= 0, SEMIPD_EINVAL, "local_attention: bad sizes");
   if (batch == 0 || num_tokens == 0) return 0;
   if (a.k_ld == 0) a.k_ld = (int64_t)num_kv_heads * qk_dim;
-  if (a.v_ld == 0) a.v_ld = (int64_t)num_kv_heads * v_dim;
+  if (a.v_ld == 0) a.v_ld = a.v_shared ? (int64_t)v_dim : (int64_t)num_kv_heads * v_dim;
   SEMIPD_CHECK_ARG(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, SEMIPD_ESHAPE,
                    "local_attention: %d query heads over %d key/value heads", num_q_heads, num_kv_heads);
   SEMIPD_CHECK_ARG(qk_dim > 0 && qk_dim <= 1024 && v_dim > 0 && v_dim <= 1024, SEMIPD_ESHAPE,
@@ -1195,24 +1290,25 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
 }
 
 extern "C" int semipd_latent_prep(const void* proj, int64_t ld, int64_t num_tokens, int num_heads, int dim, int rot_dim, int rank,
-                                  int64_t c_off, const void* norm_weight, float eps, const int64_t* positions, const float* freq,
-                                  int rot_dims, float mscale, void* pool, int64_t pool_ld, const int64_t* loc, void* q_out,
-                                  int64_t q_ld, int q_head_stride, int q_head_off, int dtype, void* stream) {
+                                  const void* latent, int64_t latent_ld, int halves, const void* norm_weight, float eps,
+                                  const int64_t* positions, const float* freq, int rot_dims, float mscale, void* pool,
+                                  int64_t pool_ld, const int64_t* loc, void* q_out, int64_t q_ld, int q_head_stride, int q_head_off,
+                                  int dtype, void* stream) {
   SEMIPD_CHECK_ARG(num_tokens >= 0 && num_heads > 0 && dim >= 0 && rot_dim >= 0 && rank > 0, SEMIPD_EINVAL, "latent_prep: bad sizes");
   if (num_tokens == 0) return 0;
   SEMIPD_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= rot_dim, SEMIPD_ESHAPE,
                    "latent_prep: %d rotated elements of a part of %d", rot_dims, rot_dim);
-  SEMIPD_CHECK_ARG(proj && norm_weight && positions && pool && loc && q_out && (freq || rot_dims == 0), SEMIPD_EINVAL,
+  SEMIPD_CHECK_ARG(proj && latent && norm_weight && positions && pool && loc && q_out && (freq || rot_dims == 0), SEMIPD_EINVAL,
                    "latent_prep: null pointer");
-  SEMIPD_CHECK_ARG(c_off >= (int64_t)num_heads * (dim + rot_dim) && ld >= c_off + rank + rot_dim && pool_ld >= rank + rot_dim &&
+  SEMIPD_CHECK_ARG(ld >= (int64_t)num_heads * (dim + rot_dim) && latent_ld >= rank + rot_dim && pool_ld >= rank + rot_dim &&
                        q_head_stride >= rot_dim && q_head_off >= 0 && q_head_off + rot_dim <= q_head_stride &&
                        q_ld >= (int64_t)num_heads * q_head_stride,
                    SEMIPD_EINVAL, "latent_prep: column ranges overlap or leave the row");
   SEMIPD_DISPATCH_DTYPE(dtype, T,
                         hipLaunchKernelGGL((latent_prep_kernel<T>), dim3((unsigned)num_tokens), dim3(256),
                                            (size_t)(rot_dims > 0 ? rot_dims : 2) * sizeof(float), as_stream(stream),
-                                           (const T*)proj, ld, num_tokens, num_heads, dim, rot_dim, rank, c_off, (const T*)norm_weight,
-                                           eps, positions, freq, rot_dims, mscale, (T*)pool, pool_ld, loc, (T*)q_out, q_ld, q_head_stride,
+                                           (const T*)proj, ld, num_tokens, num_heads, dim, rot_dim, rank, (const T*)latent, latent_ld,
+                                           halves, (const T*)norm_weight, eps, positions, freq, rot_dims, mscale, (T*)pool, pool_ld, loc, (T*)q_out, q_ld, q_head_stride,
                                            q_head_off));
   return launch_status("latent_prep");
 }
@@ -1278,4 +1374,57 @@ extern "C" int semipd_bias_rope_vnorm_kv_store(void* qkv, int64_t ld, int64_t nu
                                            (const T*)bias_q, (const T*)bias_k, (const T*)bias_v, positions, inv_freq, rot_dims,
                                            eps, (T*)k_pool, (T*)v_pool, loc));
   return launch_status("bias_rope_vnorm_kv_store");
+}
+
+
+extern "C" int semipd_qk_norm_rope_kv_store(void* qkv, int64_t ld, int64_t num_tokens, int num_q_heads, int num_kv_heads, int qk_dim,
+                                            int v_dim, int64_t k_off, int64_t v_off, const void* q_weight, const void* k_weight,
+                                            float eps, const int64_t* positions, const float* freq, int rot_dims, int halves,
+                                            float mscale, const float* head_scale, void* k_pool, void* v_pool,
+                                            const int64_t* loc, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && qk_dim > 0 && v_dim > 0, SEMIPD_EINVAL,
+                   "qk_norm_rope_kv_store: bad sizes");
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= qk_dim, SEMIPD_ESHAPE,
+                   "qk_norm_rope_kv_store: %d rotated elements of a head of %d", rot_dims, qk_dim);
+  SEMIPD_CHECK_ARG(qkv && k_pool && v_pool && loc && positions && (rot_dims == 0 || freq), SEMIPD_EINVAL,
+                   "qk_norm_rope_kv_store: null pointer");
+  SEMIPD_CHECK_ARG(k_off >= (int64_t)num_q_heads * qk_dim && v_off >= k_off + (int64_t)num_kv_heads * qk_dim &&
+                       ld >= v_off + (int64_t)num_kv_heads * v_dim,
+                   SEMIPD_EINVAL, "qk_norm_rope_kv_store: column ranges overlap or leave the row");
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((qk_norm_rope_kv_store_kernel<T>), dim3((unsigned)num_tokens), dim3(256),
+                                           (size_t)(rot_dims > 0 ? rot_dims : 2) * sizeof(float), as_stream(stream), (T*)qkv, ld,
+                                           num_q_heads, num_kv_heads, qk_dim, v_dim, k_off, v_off, (const T*)q_weight,
+                                           (const T*)k_weight, eps, positions, freq, rot_dims, halves, mscale, head_scale, (T*)k_pool,
+                                           (T*)v_pool, loc));
+  return launch_status("qk_norm_rope_kv_store");
+}
+
+// Causal softmax attention in which every query head's weights are applied to the WHOLE value row of a slot (the values of
+// all key/value heads side by side, v_row elements): out [T, heads * v_row].  Keys as in semipd_local_attention.
+extern "C" int semipd_shared_value_attention(const void* q, int64_t q_ld, void* out, int64_t out_ld, const void* k_pool,
+                                             const void* v_pool, const int32_t* req_to_token, int64_t req_to_token_stride,
+                                             const int64_t* req_pool_indices, const int64_t* seq_lens, const int32_t* q_start,
+                                             const int32_t* q_len, int64_t batch, int64_t num_tokens, int64_t max_q_len,
+                                             int num_q_heads, int num_kv_heads, int qk_dim, int v_row, float scale, int form,
+                                             int dtype, void* stream) {
+  LocalAttnArgs a{q, q_ld, nullptr, 0, out, out_ld, k_pool, v_pool, req_to_token, req_to_token_stride, req_pool_indices,
+                  seq_lens, q_start, q_len, batch, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_row, nullptr, scale, 0.f,
+                  0, 0, 0, 0, nullptr, 0, 1.0f, 0, 0, 0, nullptr, 1};
+  return launch_local_attention(a, max_q_len, form, dtype, stream);
+}
+
+extern "C" int semipd_talk_mix(const void* parts, int64_t parts_ld, const float* talk, void* out, int64_t out_ld, int64_t num_tokens,
+                               int num_q_heads, int num_kv_heads, int v_dim, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 && v_dim > 0,
+                   SEMIPD_EINVAL, "talk_mix: bad sizes");
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(parts && talk && out && parts_ld >= (int64_t)num_q_heads * num_kv_heads * v_dim &&
+                       out_ld >= (int64_t)num_q_heads * v_dim,
+                   SEMIPD_EINVAL, "talk_mix: null pointer or rows too short");
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((talk_mix_kernel<T>), dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream),
+                                           (const T*)parts, parts_ld, talk, (T*)out, out_ld, num_q_heads, num_kv_heads, v_dim));
+  return launch_status("talk_mix");
 }

@@ -165,8 +165,8 @@ _SIGNATURES = {
     "semipd_router_logits": [_vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
     "semipd_rms_stream": [_vp, _i64, _i32, _vp, _i64, _vp, _f32, _f32, _vp, _i64, _i64, _i64, _i32, _vp],
     "semipd_embed_bigram": [_vp, _vp, _vp, _f32, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i32, _vp],
-    "semipd_latent_prep": [_vp, _i64, _i64, _i32, _i32, _i32, _i32, _i64, _vp, _f32, _vp, _vp, _i32, _f32, _vp, _i64, _vp, _vp,
-                           _i64, _i32, _i32, _i32, _vp],
+    "semipd_latent_prep": [_vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _i32, _vp, _f32, _vp, _vp, _i32, _f32, _vp, _i64, _vp,
+                           _vp, _i64, _i32, _i32, _i32, _vp],
     "semipd_latent_attention": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32,
                                 _i32, _f32, _vp, _i32, _vp, _i32, _i32, _vp],
     "semipd_delta_rule": [_vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _vp, _i64,
@@ -175,10 +175,22 @@ _SIGNATURES = {
     "semipd_clamped_glu": [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _vp, _vp, _i32, _f32, _f32, _i32, _vp],
     "semipd_topk_sigmoid": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _f32, _i32, _vp],
     "semipd_sigmoid_gate": [_vp, _i64, _vp, _i64, _i64, _i64, _i32, _vp],
+    "semipd_sigmoid_gate_heads": [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _i32, _vp],
+    "semipd_embed_stream": [_vp, _vp, _f32, _i64, _vp, _i64, _i32, _vp],
+    "semipd_postnorm_stream": [_vp, _i64, _vp, _vp, _i64, _f32, _vp, _f32, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i32, _vp],
+    "semipd_token_shift": [_vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _vp],
+    "semipd_qk_norm_rope_kv_store": [_vp, _i64, _i64, _i32, _i32, _i32, _i32, _i64, _i64, _vp, _vp, _f32, _vp, _vp, _i32, _i32, _f32,
+                                     _vp, _vp, _vp, _vp, _i32, _vp],
+    "semipd_shared_value_attention": [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32,
+                                      _i32, _i32, _f32, _i32, _i32, _vp],
+    "semipd_talk_mix": [_vp, _i64, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
+    "semipd_state_space_work_width": [_i32, _i32, _i32, _i32],
+    "semipd_state_space": [_vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _vp, _i64, _vp, _i64, _vp, _i64,
+                           _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _i64, _i32, _i32, _vp],
 }
 _RESTYPES = {"semipd_last_error": C.c_char_p, "semipd_lm_head_argmax_workspace": _sz,
              "semipd_linear_workspace": _sz, "semipd_stream_linear_workspace": _sz, "semipd_dense_gemm_report": _sz, "semipd_ar_meta_size": _sz, "semipd_ar_region_size": _sz,
-             "semipd_min_gru_workspace": _i64, "semipd_delta_rule_work_width": _i64}
+             "semipd_min_gru_workspace": _i64, "semipd_delta_rule_work_width": _i64, "semipd_state_space_work_width": _i64}
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
@@ -193,6 +205,7 @@ MODEL_SOURCES = {
     "Kudirax": ("local_attention.hip", "layernorm.hip"),
     "Tigotar": ("local_attention.hip", "layernorm.hip", "recurrent.hip"),
     "Penozen": ("local_attention.hip", "layernorm.hip", "delta_rule.hip"),
+    "Tibenex": ("local_attention.hip", "layernorm.hip", "state_space.hip"),
 }
 
 

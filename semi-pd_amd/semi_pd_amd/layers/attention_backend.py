@@ -333,6 +333,31 @@ class HipAttnBackend(AttentionBackend):
             kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
         return o
 
+    # ---- every head's weights over the values of ALL key/value heads (the input of a mix of the heads' weights) ------------
+    def forward_shared_values(self, q, layer, forward_batch: ForwardBatch):
+        """Causal softmax attention for layers whose keys and values are in the pool already, in which every query head's
+        weights are applied to the values of all key/value heads: q [T, heads * head_dim] (may be a column range) ->
+        [T, heads * kv_heads * v_head_dim], head h's block holding its weights applied to key/value head 0, 1, ...  Keys:
+        head h reads key head h / (heads / kv_heads).  One call for prompt portions, single tokens and decode batches."""
+        T = q.shape[0]
+        G = layer.tp_k_head_num
+        o = torch.empty((T, layer.tp_q_head_num * G * layer.v_head_dim), dtype=q.dtype, device=q.device)
+        pool = forward_batch.token_to_kv_pool
+        if forward_batch.forward_mode.is_decode():
+            q_start = q_len = None
+            max_q = 1
+        else:
+            q_start, q_len = forward_batch.extend_start_loc, forward_batch.extend_seq_lens
+            max_q = max(forward_batch.extend_seq_lens_cpu)
+        kt = self._timing()
+        t0 = kt.start() if kt else None
+        ops.shared_value_attention_fwd(q, o, pool.get_key_buffer(layer.layer_id), pool.get_value_buffer(layer.layer_id),
+                                       self.req_to_token, forward_batch.req_pool_indices, forward_batch.seq_lens, q_start, q_len,
+                                       max_q, layer.scaling, form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")))
+        if kt:
+            kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
+        return o
+
     # ---- decode: RoPE + KV store + attention + split merge in one launch -------------------------
     def fused_decode_waves(self, bs: int, head_dim: int, num_kv_splits: int = 0) -> int:
         """How a decode batch of `bs` requests goes from the qkv GEMM's planes to o_proj's input: 0 = the separate

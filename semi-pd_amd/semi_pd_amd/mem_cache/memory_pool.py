@@ -183,8 +183,12 @@ class MHATokenToKVPool:
         self.head_nums, self.head_dims = per_layer(head_num), per_layer(head_dim)
         self.v_head_dims = per_layer(v_head_dim) if v_head_dim is not None else list(self.head_dims)
         assert len(self.head_nums) == len(self.head_dims) == len(self.v_head_dims) == layer_num
-        self.values_in_keys = bool(values_in_keys)
-        if self.values_in_keys and any(h != 1 or dv > d for h, d, dv in zip(self.head_nums, self.head_dims, self.v_head_dims)):
+        # per layer (a model may have both kinds of layers); one flag stands for every layer
+        self.in_keys = [bool(v) for v in values_in_keys] if isinstance(values_in_keys, (list, tuple)) \
+            else [bool(values_in_keys)] * layer_num
+        assert len(self.in_keys) == layer_num
+        self.values_in_keys = any(self.in_keys)
+        if any(f and (h != 1 or dv > d) for f, h, d, dv in zip(self.in_keys, self.head_nums, self.head_dims, self.v_head_dims)):
             raise ValueError("values_in_keys: one key/value head per layer whose values are a prefix of its key rows")
         self.uniform = (len(set(self.head_nums)) == 1 and len(set(self.head_dims)) == 1
                         and self.v_head_dims == self.head_dims and not self.values_in_keys)
@@ -198,11 +202,11 @@ class MHATokenToKVPool:
     def _regions(self):
         """(key offset, value offset) in bytes of every layer inside the byte slab, and the slab's size."""
         rows, es, off, out = self.size + self.page_size, self.dtype.itemsize, 0, []
-        for h, d, dv in zip(self.head_nums, self.head_dims, self.v_head_dims):
+        for h, d, dv, in_keys in zip(self.head_nums, self.head_dims, self.v_head_dims, self.in_keys):
             k_off = off
             off = -(-(off + rows * h * d * es) // 256) * 256
             v_off = off
-            if not self.values_in_keys:
+            if not in_keys:
                 off = -(-(off + rows * h * dv * es) // 256) * 256
             out.append((k_off, v_off))
         return out, off
@@ -218,21 +222,23 @@ class MHATokenToKVPool:
         regions, total = self._regions()
         self.slab = ipc_safe_zeros((total,), torch.uint8, self.device)
         rows, es = self.size + self.page_size, self.dtype.itemsize
-        for (k_off, v_off), h, d, dv in zip(regions, self.head_nums, self.head_dims, self.v_head_dims):
+        for (k_off, v_off), h, d, dv, in_keys in zip(regions, self.head_nums, self.head_dims, self.v_head_dims, self.in_keys):
             self.k_buffer.append(self.slab[k_off: k_off + rows * h * d * es].view(self.dtype).view(rows, h, d))
-            if not self.values_in_keys:
-                self.v_buffer.append(self.slab[v_off: v_off + rows * h * dv * es].view(self.dtype).view(rows, h, dv))
+            self.v_buffer.append(None if in_keys
+                                 else self.slab[v_off: v_off + rows * h * dv * es].view(self.dtype).view(rows, h, dv))
         self.link_value_views()
 
     def link_value_views(self):
         """values_in_keys: the value buffers as views of the key buffers (after creating them or mapping them from another process)."""
         if self.values_in_keys:
-            self.v_buffer = [k[..., :dv] for k, dv in zip(self.k_buffer, self.v_head_dims)]
+            have = list(self.v_buffer) + [None] * (self.layer_num - len(self.v_buffer))
+            self.v_buffer = [k[..., :dv] if in_keys else v
+                             for k, v, dv, in_keys in zip(self.k_buffer, have, self.v_head_dims, self.in_keys)]
 
     def get_kv_size_bytes(self):
         rows, es = self.size + self.page_size, self.dtype.itemsize
         k = sum(rows * h * d * es for h, d in zip(self.head_nums, self.head_dims))
-        v = 0 if self.values_in_keys else sum(rows * h * d * es for h, d in zip(self.head_nums, self.v_head_dims))
+        v = sum(0 if f else rows * h * d * es for h, d, f in zip(self.head_nums, self.v_head_dims, self.in_keys))
         return k, v
 
     def get_key_buffer(self, layer_id: int):

@@ -54,6 +54,9 @@ def build_model(model_config, dtype):
     if arch == "Penozen":
         from semi_pd_amd.models.penozen import PenozenForCausalLM
         return PenozenForCausalLM(model_config, dtype)
+    if arch == "Tibenex":
+        from semi_pd_amd.models.tibenex import TibenexForCausalLM
+        return TibenexForCausalLM(model_config, dtype)
     raise ValueError(f"unsupported architecture {arch}")
 
 
@@ -293,8 +296,11 @@ class ModelRunner:
         if geo["kind"] == "mla":
             cell = (geo["kv_lora_rank"] + geo["qk_rope_head_dim"]) * geo["num_layers"] * self.kv_cache_dtype.itemsize
         elif isinstance(geo["num_kv_heads"], (list, tuple)):
-            in_keys = bool(geo.get("values_in_keys"))       # values that are a prefix of the key rows take no room of their own
-            cell = sum(h * (d + (0 if in_keys else dv)) for h, d, dv in zip(geo["num_kv_heads"], geo["head_dim"], geo["v_head_dim"])) \
+            in_keys = geo.get("values_in_keys")       # values that are a prefix of the key rows take no room of their own
+            if not isinstance(in_keys, (list, tuple)):
+                in_keys = [bool(in_keys)] * len(geo["num_kv_heads"])
+            cell = sum(h * (d + (0 if f else dv))
+                       for h, d, dv, f in zip(geo["num_kv_heads"], geo["head_dim"], geo["v_head_dim"], in_keys)) \
                 * self.kv_cache_dtype.itemsize
         else:
             cell = (geo["num_kv_heads"] * (geo["head_dim"] + geo["v_head_dim"]) * geo["num_layers"]
@@ -327,7 +333,7 @@ class ModelRunner:
             self.token_to_kv_pool = MHATokenToKVPool(self.max_total_num_tokens, 1, self.kv_cache_dtype,
                                                      geo["num_kv_heads"], geo["head_dim"], geo["num_layers"],
                                                      dev, bypass_create_buffers=bypass, v_head_dim=geo["v_head_dim"],
-                                                     values_in_keys=bool(geo.get("values_in_keys")))
+                                                     values_in_keys=geo.get("values_in_keys") or False)
         self.token_to_kv_pool_allocator = TokenToKVPoolAllocator(self.max_total_num_tokens, self.kv_cache_dtype, dev,
                                                                  self.token_to_kv_pool)
         # models with recurrent layers: one fp32 state row per running request (`state_geometry`: the width of every
@@ -385,7 +391,7 @@ class ModelRunner:
             for i in range(pool.layer_num):
                 # (values that are views of the key rows travel with the keys' handle)
                 kv_handles.append([get_ipc_handle(pool.k_buffer[i]),
-                                   None if pool.values_in_keys else get_ipc_handle(pool.v_buffer[i])])
+                                   None if pool.in_keys[i] else get_ipc_handle(pool.v_buffer[i])])
             kv_info = {"kind": "mha", "shape": tuple(pool.k_buffer[0].shape), "dtype": pool.dtype,
                        "numel": pool.k_buffer[0].numel(), "layer_num": pool.layer_num}
             if not pool.uniform:
@@ -458,10 +464,9 @@ class ModelRunner:
                     n *= d
                 return self._import(handle, {"numel": n, "dtype": kvi["dtype"], "shape": tuple(shape), "contiguous": True})
             pool.k_buffer = [one(h[0], sh[0]) for h, sh in zip(ipc_info.kv_cache_handles, kvi["shapes"])]
+            pool.v_buffer = [None if h[1] is None else one(h[1], sh[1]) for h, sh in zip(ipc_info.kv_cache_handles, kvi["shapes"])]
             if pool.values_in_keys:
                 pool.link_value_views()
-            else:
-                pool.v_buffer = [one(h[1], sh[1]) for h, sh in zip(ipc_info.kv_cache_handles, kvi["shapes"])]
         elif kvi["kind"] == "mha":
             pool.k_buffer = [self._import(h[0], info) for h in ipc_info.kv_cache_handles]
             pool.v_buffer = [self._import(h[1], info) for h in ipc_info.kv_cache_handles]

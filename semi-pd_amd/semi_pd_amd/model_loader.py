@@ -28,8 +28,9 @@ def _config_classes():
     from semi_pd_amd.models.kudirax import KudiraxConfig
     from semi_pd_amd.models.opt import OPTConfig
     from semi_pd_amd.models.penozen import PenozenConfig
+    from semi_pd_amd.models.tibenex import TibenexConfig
     from semi_pd_amd.models.tigotar import TigotarConfig
-    return {"Tigotar": TigotarConfig, "Penozen": PenozenConfig, "LlamaForCausalLM": LlamaConfig, "OPTForCausalLM": OPTConfig,
+    return {"Tibenex": TibenexConfig, "Tigotar": TigotarConfig, "Penozen": PenozenConfig, "LlamaForCausalLM": LlamaConfig, "OPTForCausalLM": OPTConfig,
             "DeepseekV2ForCausalLM": DeepseekV2Config, "DeepseekV3ForCausalLM": DeepseekV2Config,
             "Kudirax": KudiraxConfig}
 
@@ -280,6 +281,77 @@ def _penozen_items(config, weights):
         raise RuntimeError(f"checkpoint ended with incomplete stacked parameters: {list(st.pending)[:4]}")
 
 
+_TIBENEX_RE = re.compile(r"^l(\d+)\.(mix|mlp|norm1|norm2|ls1|ls2|shift)(?:\.(.+))?$")
+_TIBENEX_LATENT_IN = {"dq": 0, "dkv": 1, "g": 2}
+_TIBENEX_LATENT_LEAF = {"dq.norm": "q_norm", "uq": "q_up", "dkv.norm": "latent_norm", "o": "out_proj.weight"}
+_TIBENEX_ATTN_IN = {"q": 0, "k": 1, "v": 2}
+_TIBENEX_ATTN_LEAF = {"q.norm": "q_norm", "k.norm": "k_norm", "talk": "talk", "temp": "temp", "o": "out_proj.weight"}
+_TIBENEX_SSM_LEAF = {"in": "in_proj.weight", "conv": "conv", "conv.b": "conv_bias", "dt_bias": "dt_bias", "A_log": "a_log", "D": "d_skip",
+                     "norm": "out_norm", "o": "out_proj.weight"}
+_TIBENEX_SEAM = {"norm1": "norm1.weight", "norm2": "norm2.weight", "ls1": "norm1.layer_scale", "ls2": "norm2.layer_scale",
+                 "shift": "shift.mu"}
+
+
+def _tibenex_items(config, weights):
+    """Tibenex checkpoint names (embed, l<i>.norm1|norm2|ls1|ls2|shift, l<i>.mix.dq|dq.norm|uq|dkv|dkv.norm|uk|uv|g|o of a
+    latent-attention layer, l<i>.mix.q|k|v|q.norm|k.norm|talk|temp|o of an attention layer, l<i>.mix.in|conv|conv.b|dt_bias|
+    A_log|D|norm|o of a state-space layer, l<i>.mlp.gate|up|down, final.norm, head) -> product parameters: dq | dkv | g
+    (q | k | v) stack into the mixer's merged input projection, the up-projections of keys and values are cut by head, gate
+    and up stack into the feed-forward's merged projection."""
+    st = _Stacker()
+    top = {"embed": "embed.weight", "head": "head.weight", "final.norm": "final_norm_weight"}
+    for name, t in weights:
+        if name in top:
+            yield top[name], t
+            continue
+        m = _TIBENEX_RE.match(name)
+        if not m or int(m.group(1)) >= len(config.layers):
+            raise KeyError(f"checkpoint tensor {name} has no counterpart in a Tibenex model")
+        i, part, leaf = int(m.group(1)), m.group(2), m.group(3)
+        base = f"layers.{i}."
+        lc = config.layers[i]
+        if part in _TIBENEX_SEAM:
+            if leaf is not None:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Tibenex model")
+            if part in ("norm2", "ls2") and not lc.ff:
+                continue                      # a layer without feed-forward has no second sum to norm
+            yield base + _TIBENEX_SEAM[part], t
+        elif part == "mix" and lc.kind == "latent_attention":
+            mc = lc.mixer
+            if leaf in _TIBENEX_LATENT_IN:
+                yield from st.add(base + "mix.in_proj.weight", _TIBENEX_LATENT_IN[leaf], 3, t)
+            elif leaf in _TIBENEX_LATENT_LEAF:
+                yield base + "mix." + _TIBENEX_LATENT_LEAF[leaf], t
+            elif leaf == "uk":
+                yield base + "mix.w_uk", t.reshape(mc.heads, mc.dim, mc.kv_rank)
+            elif leaf == "uv":
+                yield base + "mix.w_uv", t.reshape(mc.heads, mc.vdim, mc.kv_rank)
+            else:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a latent-attention layer")
+        elif part == "mix" and lc.kind == "attention":
+            if leaf in _TIBENEX_ATTN_IN:
+                yield from st.add(base + "mix.in_proj.weight", _TIBENEX_ATTN_IN[leaf], 3, t)
+            elif leaf in _TIBENEX_ATTN_LEAF:
+                yield base + "mix." + _TIBENEX_ATTN_LEAF[leaf], t
+            else:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in an attention layer")
+        elif part == "mix":
+            if leaf not in _TIBENEX_SSM_LEAF:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a state-space layer")
+            yield base + "mix." + _TIBENEX_SSM_LEAF[leaf], t
+        else:
+            if not lc.ff:
+                raise KeyError(f"checkpoint tensor {name}: layer {i} has no feed-forward")
+            if leaf in ("gate", "up"):
+                yield from st.add(base + "mlp.gate_up_proj.weight", int(leaf == "up"), 2, t)
+            elif leaf == "down":
+                yield base + "mlp.down_proj.weight", t
+            else:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Tibenex model")
+    if st.pending:
+        raise RuntimeError(f"checkpoint ended with incomplete stacked parameters: {list(st.pending)[:4]}")
+
+
 _EXPERT_RE = re.compile(r"^(.*\.mlp\.experts)\.(\d+)\.(gate_proj|up_proj|down_proj)\.(weight|weight_scale_inv)$")
 
 
@@ -294,6 +366,9 @@ def product_items(config, weights: Iterable[Tuple[str, torch.Tensor]]) -> Iterat
         return
     if arch == "Penozen":
         yield from _penozen_items(config, weights)
+        return
+    if arch == "Tibenex":
+        yield from _tibenex_items(config, weights)
         return
     st = _Stacker()
     tie = bool(getattr(config, "tie_word_embeddings", False))

@@ -250,8 +250,9 @@ class PenozenLatentAttention(nn.Module):
         T = p.shape[0]
         pool = forward_batch.token_to_kv_pool.get_key_buffer(self.attn.layer_id)
         pool = pool.view(pool.shape[0], -1)
-        ops.latent_prep(p, H, D, P, R, self.q_size, self.latent_norm, self.eps, forward_batch.positions,
-                        self.freq if mc.rot_dims else None, mc.rot_dims, self.mscale, pool, forward_batch.out_cache_loc)
+        ops.latent_prep(p, p[:, self.q_size: self.q_size + self.c_size], H, D, P, R, self.latent_norm, self.eps,
+                        forward_batch.positions, self.freq if mc.rot_dims else None, mc.rot_dims, self.mscale, pool,
+                        forward_batch.out_cache_loc)
         slots, table, rows = context_rows(forward_batch)
         ctx = ops.gather_rows(pool, slots)                                    # [N, R + P]: every request's tokens, in order
         keys = dense_linear(ctx, self.w_key_rows)                             # [N, H * (D + P)]
@@ -272,9 +273,9 @@ class PenozenLatentAttention(nn.Module):
             return self._forward_expanded(p, forward_batch)
         pool = forward_batch.token_to_kv_pool.get_key_buffer(self.attn.layer_id)
         q_in = torch.empty((T, H * (R + P)), dtype=p.dtype, device=p.device)
-        ops.latent_prep(p, H, D, P, R, self.q_size, self.latent_norm, self.eps, forward_batch.positions,
-                        self.freq if mc.rot_dims else None, mc.rot_dims, self.mscale, pool.view(pool.shape[0], -1),
-                        forward_batch.out_cache_loc, q_in)
+        ops.latent_prep(p, p[:, self.q_size: self.q_size + self.c_size], H, D, P, R, self.latent_norm, self.eps,
+                        forward_batch.positions, self.freq if mc.rot_dims else None, mc.rot_dims, self.mscale,
+                        pool.view(pool.shape[0], -1), forward_batch.out_cache_loc, q_in)
         # the unrotated query part through the key up-projection, head by head: [H, T, D] x [H, D, R] -> q_in[:, h, :R]
         q_u = p[:, : self.q_size].view(T, H, D + P)[..., :D]
         torch.bmm(q_u.transpose(0, 1), self.w_uk, out=q_in.view(T, H, R + P)[..., :R].transpose(0, 1))

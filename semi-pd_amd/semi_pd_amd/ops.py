@@ -1642,16 +1642,20 @@ def embed_bigram(input_ids: torch.Tensor, embed: torch.Tensor, bigram: torch.Ten
     return out
 
 
-def latent_prep(proj: torch.Tensor, num_heads: int, dim: int, rot_dim: int, rank: int, c_off: int, norm_weight: torch.Tensor,
+def latent_prep(proj: torch.Tensor, latent: torch.Tensor, num_heads: int, dim: int, rot_dim: int, rank: int, norm_weight: torch.Tensor,
                 eps: float, positions: torch.Tensor, freq: Optional[torch.Tensor], rot_dims: int, mscale: float,
-                pool: torch.Tensor, loc: torch.Tensor, q_out: Optional[torch.Tensor] = None) -> None:
-    """Rows of `proj`: per head [dim | rot_dim] query elements from column 0, the latent [rank] and the shared rotated key
-    part [rot_dim] at column c_off.  pool[loc] <- [rms_norm(latent) * norm_weight | key part turned by the position];
-    q_out [T, heads * (rank + rot_dim)]: every head's last rot_dim elements <- its rotated query part turned; without q_out
-    the rotated query parts are turned in place (csrc/local_attention.hip: semipd_latent_prep)."""
+                pool: torch.Tensor, loc: torch.Tensor, q_out: Optional[torch.Tensor] = None, halves: bool = False) -> None:
+    """Rows of `proj`: per head [dim | rot_dim] query elements from column 0; rows of `latent` (a column range of the same
+    projection, or another projection's rows): the latent [rank] and the shared rotated key part [rot_dim].
+    pool[loc] <- [rms_norm(latent) * norm_weight | key part turned by the position]; q_out [T, heads * (rank + rot_dim)]: every
+    head's last rot_dim elements <- its rotated query part turned; without q_out the rotated query parts are turned in place.
+    Pair i of a rotation is elements (2i, 2i + 1), with `halves` (i, i + rot_dims / 2) (csrc/local_attention.hip:
+    semipd_latent_prep)."""
     T = proj.shape[0]
-    if proj.dim() != 2 or proj.stride(1) != 1:
-        raise RuntimeError("latent_prep: proj is 2-D with contiguous rows")
+    if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < num_heads * (dim + rot_dim):
+        raise RuntimeError("latent_prep: proj is [T, >= heads * (dim + rot_dim)] with contiguous rows")
+    if latent.dim() != 2 or latent.stride(1) != 1 or latent.dtype != proj.dtype or latent.shape != (T, rank + rot_dim):
+        raise RuntimeError("latent_prep: latent is [T, rank + rot_dim] of the activation type with contiguous rows")
     if q_out is None:
         q_out, stride, off = proj, dim + rot_dim, dim
     else:
@@ -1666,10 +1670,10 @@ def latent_prep(proj: torch.Tensor, num_heads: int, dim: int, rot_dim: int, rank
         raise RuntimeError("latent_prep: norm_weight is contiguous [rank] of the activation type")
     if rot_dims and (freq is None or freq.dtype != torch.float32 or freq.numel() != rot_dims // 2 or not freq.is_contiguous()):
         raise RuntimeError("latent_prep: freq is fp32 [rot_dims / 2]")
-    check(_lib.load().semipd_latent_prep(ptr(proj), proj.stride(0), T, num_heads, dim, rot_dim, rank, int(c_off), ptr(norm_weight),
-                                         float(eps), ptr(positions), ptr(freq), int(rot_dims), float(mscale), ptr(pool),
-                                         pool.stride(0), ptr(loc), ptr(q_out), q_out.stride(0), stride, off, dtype_code(proj.dtype),
-                                         current_stream(proj.device)), "latent_prep")
+    check(_lib.load().semipd_latent_prep(ptr(proj), proj.stride(0), T, num_heads, dim, rot_dim, rank, ptr(latent), latent.stride(0),
+                                         1 if halves else 0, ptr(norm_weight), float(eps), ptr(positions), ptr(freq), int(rot_dims),
+                                         float(mscale), ptr(pool), pool.stride(0), ptr(loc), ptr(q_out), q_out.stride(0), stride, off,
+                                         dtype_code(proj.dtype), current_stream(proj.device)), "latent_prep")
 
 
 def latent_attention_fwd(q: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, rank: int, req_to_token: torch.Tensor,
@@ -1792,3 +1796,220 @@ def sigmoid_gate_(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
     check(_lib.load().semipd_sigmoid_gate(ptr(x), x.stride(0), ptr(gate), gate.stride(0), x.shape[0], x.shape[1],
                                           dtype_code(x.dtype), current_stream(x.device)), "sigmoid_gate")
     return x
+
+
+# ---- norm after the sum on an fp32 stream, token shift, attention whose heads talk, state-space recurrence -----------------
+def sigmoid_gate_heads_(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """x [rows, heads * size] <- x * sigmoid(gate [rows, heads]) in place, one gate per head, fp32 arithmetic
+    (csrc/layernorm.hip); rows may be column ranges of wider rows."""
+    if x.dim() != 2 or gate.dim() != 2 or x.shape[0] != gate.shape[0] or x.dtype != gate.dtype or x.stride(1) != 1 \
+            or gate.stride(1) != 1 or gate.shape[1] == 0 or x.shape[1] % gate.shape[1]:
+        raise RuntimeError("sigmoid_gate_heads_: x [rows, heads * size] and gate [rows, heads] of one type with contiguous rows")
+    check(_lib.load().semipd_sigmoid_gate_heads(ptr(x), x.stride(0), ptr(gate), gate.stride(0), x.shape[0], gate.shape[1],
+                                                x.shape[1] // gate.shape[1], dtype_code(x.dtype), current_stream(x.device)),
+          "sigmoid_gate_heads")
+    return x
+
+
+def embed_stream(input_ids: torch.Tensor, embed: torch.Tensor, scale: float) -> torch.Tensor:
+    """fp32 [T, width] = embed[id] * scale: the start of an fp32 residual stream (csrc/layernorm.hip)."""
+    if input_ids.dtype != torch.int64 or not input_ids.is_contiguous() or embed.dim() != 2 or not embed.is_contiguous():
+        raise RuntimeError("embed_stream: int64 ids, embed [V, W] contiguous")
+    out = torch.empty((input_ids.shape[0], embed.shape[1]), dtype=torch.float32, device=embed.device)
+    check(_lib.load().semipd_embed_stream(ptr(input_ids), ptr(embed), float(scale), input_ids.shape[0], ptr(out), embed.shape[1],
+                                          dtype_code(embed.dtype), current_stream(embed.device)), "embed_stream")
+    return out
+
+
+def postnorm_stream(y: Optional[torch.Tensor], layer_scale: Optional[torch.Tensor], stream: torch.Tensor, alpha: float,
+                    weight: torch.Tensor, eps: float, want_out: bool = True, shift_mu: Optional[torch.Tensor] = None,
+                    prev: Optional[torch.Tensor] = None, state_indices: Optional[torch.Tensor] = None,
+                    seq_lens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """stream (fp32 [rows, width], in place) <- rms_norm(alpha * stream + layer_scale * y) * weight, the norm AFTER the sum.
+    Returns the new stream in the weight's type (None with want_out=False); with shift_mu -- batches of one row per request
+    -- the token-shifted stream s + (prev[state_indices] - s) * shift_mu instead, prev (fp32 [slots, width], a column range of
+    the requests' state rows; zeros where seq_lens <= 1) then taking s (csrc/layernorm.hip: semipd_postnorm_stream)."""
+    if stream.dim() != 2 or stream.dtype != torch.float32 or stream.stride(1) != 1:
+        raise RuntimeError("postnorm_stream: the stream is fp32 [rows, width] with contiguous rows")
+    rows, width = stream.shape
+    dt = weight.dtype
+    if weight.shape != (width,) or not weight.is_contiguous():
+        raise RuntimeError("postnorm_stream: weight is contiguous [width]")
+    if y is not None and (y.shape != stream.shape or y.stride(1) != 1 or y.dtype != dt):
+        raise RuntimeError("postnorm_stream: y is shaped like the stream, of the weight's type")
+    if layer_scale is not None and (layer_scale.shape != (width,) or layer_scale.dtype != dt or not layer_scale.is_contiguous()):
+        raise RuntimeError("postnorm_stream: layer_scale is contiguous [width] of the weight's type")
+    if shift_mu is not None:
+        if not want_out or shift_mu.shape != (width,) or shift_mu.dtype != dt or not shift_mu.is_contiguous():
+            raise RuntimeError("postnorm_stream: shift_mu is contiguous [width] of the weight's type and needs the output")
+        if prev is None or prev.dtype != torch.float32 or prev.dim() != 2 or prev.shape[1] != width or prev.stride(1) != 1:
+            raise RuntimeError("postnorm_stream: prev is fp32 [slots, width]")
+        if state_indices is None or seq_lens is None or state_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64 \
+                or state_indices.shape[0] != rows or seq_lens.shape[0] != rows:
+            raise RuntimeError("postnorm_stream: the shifted form takes one row per request: state_indices / seq_lens int64 [rows]")
+    out = torch.empty((rows, width), dtype=dt, device=stream.device) if want_out else None
+    check(_lib.load().semipd_postnorm_stream(ptr(y), y.stride(0) if y is not None else 0, ptr(layer_scale), ptr(stream),
+                                             stream.stride(0), float(alpha), ptr(weight), float(eps), ptr(out),
+                                             out.stride(0) if out is not None else 0, ptr(shift_mu), ptr(prev),
+                                             prev.stride(0) if prev is not None else 0, ptr(state_indices), ptr(seq_lens), rows, width,
+                                             dtype_code(dt), current_stream(stream.device)), "postnorm_stream")
+    return out
+
+
+def token_shift(stream: torch.Tensor, mu: torch.Tensor, prev: torch.Tensor, state_indices: torch.Tensor, seq_lens: torch.Tensor,
+                q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor]) -> torch.Tensor:
+    """[T, width] of mu's type = s_t + (s_(t-1) - s_t) * mu over the fp32 stream s; the row in front of a request's rows is its
+    entry of prev (fp32 [slots, width], a column range of the requests' state rows; zeros at position 0), and the request's
+    last row is left there (csrc/layernorm.hip: semipd_token_shift)."""
+    if stream.dim() != 2 or stream.dtype != torch.float32 or stream.stride(1) != 1:
+        raise RuntimeError("token_shift: the stream is fp32 [T, width] with contiguous rows")
+    T, width = stream.shape
+    B = state_indices.shape[0]
+    if mu.shape != (width,) or not mu.is_contiguous():
+        raise RuntimeError("token_shift: mu is contiguous [width]")
+    if prev.dtype != torch.float32 or prev.dim() != 2 or prev.shape[1] != width or prev.stride(1) != 1:
+        raise RuntimeError("token_shift: prev is fp32 [slots, width]")
+    if state_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64 or seq_lens.shape[0] != B:
+        raise RuntimeError("token_shift: state_indices / seq_lens are int64 [B]")
+    _batch_rows("token_shift", T, B, q_start, q_len)
+    out = torch.empty((T, width), dtype=mu.dtype, device=stream.device)
+    check(_lib.load().semipd_token_shift(ptr(stream), stream.stride(0), ptr(mu), ptr(prev), prev.stride(0), ptr(state_indices),
+                                         ptr(seq_lens), ptr(q_start), ptr(q_len), B, T, ptr(out), out.stride(0), width,
+                                         dtype_code(mu.dtype), current_stream(stream.device)), "token_shift")
+    return out
+
+
+def qk_norm_rope_kv_store(qkv: torch.Tensor, num_q_heads: int, num_kv_heads: int, qk_dim: int, v_dim: int, k_off: int, v_off: int,
+                          q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float, positions: torch.Tensor,
+                          freq: Optional[torch.Tensor], rot_dims: int, halves: bool, mscale: float,
+                          head_scale: Optional[torch.Tensor], k_buffer: torch.Tensor, v_buffer: torch.Tensor,
+                          loc: torch.Tensor) -> None:
+    """Rows of `qkv` hold q | k | v at columns 0, k_off, v_off: q and k normed over the whole projection (all heads at once)
+    times q_weight / k_weight, the first rot_dims elements of every head turned by positions * freq (pairs (2i, 2i + 1), with
+    `halves` (i, i + rot_dims / 2); cos and sin times mscale), query head h times head_scale[h]; q in place, k / v into the pools at `loc`
+    (csrc/local_attention.hip)."""
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise RuntimeError("qk_norm_rope_kv_store: qkv must be 2-D with contiguous rows")
+    T = qkv.shape[0]
+    if loc.dtype != torch.int64 or positions.dtype != torch.int64 or loc.shape[0] != T or positions.shape[0] != T:
+        raise RuntimeError("qk_norm_rope_kv_store: one int64 pool slot and position per row")
+    for buf, size, name in ((k_buffer, qk_dim, "k_buffer"), (v_buffer, v_dim, "v_buffer")):
+        if buf.dtype != qkv.dtype or buf.dim() != 3 or buf.shape[1] != num_kv_heads or buf.shape[2] != size \
+                or not buf.is_contiguous():
+            raise RuntimeError(f"qk_norm_rope_kv_store: {name} must be a contiguous [N, {num_kv_heads}, {size}] pool of {qkv.dtype}")
+    for w_, n in ((q_weight, num_q_heads * qk_dim), (k_weight, num_kv_heads * qk_dim)):
+        if w_ is not None and (w_.shape != (n,) or w_.dtype != qkv.dtype or not w_.is_contiguous()):
+            raise RuntimeError("qk_norm_rope_kv_store: norm weights are contiguous [heads * size] of the activation type")
+    if head_scale is not None and (head_scale.dtype != torch.float32 or head_scale.shape != (num_q_heads,)
+                                   or not head_scale.is_contiguous()):
+        raise RuntimeError("qk_norm_rope_kv_store: head_scale is fp32 [heads]")
+    if rot_dims and (freq is None or freq.dtype != torch.float32 or freq.numel() != rot_dims // 2 or not freq.is_contiguous()):
+        raise RuntimeError("qk_norm_rope_kv_store: freq is fp32 [rot_dims / 2]")
+    check(_lib.load().semipd_qk_norm_rope_kv_store(ptr(qkv), qkv.stride(0), T, num_q_heads, num_kv_heads, qk_dim, v_dim, int(k_off),
+                                                   int(v_off), ptr(q_weight), ptr(k_weight), float(eps), ptr(positions), ptr(freq),
+                                                   int(rot_dims), 1 if halves else 0, float(mscale), ptr(head_scale), ptr(k_buffer), ptr(v_buffer),
+                                                   ptr(loc), dtype_code(qkv.dtype), current_stream(qkv.device)),
+          "qk_norm_rope_kv_store")
+
+
+def shared_value_attention_fwd(q: torch.Tensor, out: torch.Tensor, k_buffer: torch.Tensor, v_buffer: torch.Tensor,
+                               req_to_token: torch.Tensor, req_pool_indices: torch.Tensor, seq_lens: torch.Tensor,
+                               q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor], max_q_len: int, sm_scale: float,
+                               form: int = 0) -> None:
+    """Causal softmax attention over the paged pools in which every query head's weights are applied to the values of ALL
+    key/value heads: q [T, H * D], keys [N, G, D] (head h reads key head h / (H / G)), values [N, G, E] read as one row of
+    G * E elements, out [T, H * G * E].  Batch description as in local_attention_fwd (csrc/local_attention.hip)."""
+    T = q.shape[0]
+    G, D = k_buffer.shape[1], k_buffer.shape[2]
+    row = v_buffer.shape[1] * v_buffer.shape[2]
+    if q.dim() != 2 or out.dim() != 2 or q.stride(1) != 1 or out.stride(1) != 1 or q.shape[1] % D:
+        raise RuntimeError("shared_value_attention_fwd: q / out are [T, heads * size] with contiguous rows")
+    H = q.shape[1] // D
+    if out.shape != (T, H * row) or out.dtype != q.dtype or k_buffer.dtype != q.dtype or v_buffer.dtype != q.dtype:
+        raise RuntimeError("shared_value_attention_fwd: shapes or types of q, out and the pools disagree")
+    if not (k_buffer.is_contiguous() and v_buffer.is_contiguous()) or v_buffer.shape[1] != G or H % G:
+        raise RuntimeError("shared_value_attention_fwd: pools must be contiguous [N, G, size], heads a multiple of G")
+    if req_to_token.dtype != torch.int32 or req_pool_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64:
+        raise RuntimeError("shared_value_attention_fwd: req_to_token int32, req_pool_indices / seq_lens int64")
+    B = req_pool_indices.shape[0]
+    _batch_rows("shared_value_attention_fwd", T, B, q_start, q_len)
+    check(_lib.load().semipd_shared_value_attention(ptr(q), q.stride(0), ptr(out), out.stride(0), ptr(k_buffer), ptr(v_buffer),
+                                                    ptr(req_to_token), req_to_token.stride(0), ptr(req_pool_indices), ptr(seq_lens),
+                                                    ptr(q_start), ptr(q_len), B, T, int(max_q_len), H, G, D, row, float(sm_scale),
+                                                    int(form), dtype_code(q.dtype), current_stream(q.device)),
+          "shared_value_attention")
+
+
+def talk_mix(parts: torch.Tensor, talk: torch.Tensor, num_kv_heads: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out [T, H * E]: out[t, h] = sum_g talk[h, g] * parts[t, g, c(h)], parts [T, H * G * E] the weights of head g applied to
+    the values of key/value head c, c(h) = h / (H / G): the heads' attention weights mixed after the softmax
+    (csrc/local_attention.hip: semipd_talk_mix)."""
+    H = talk.shape[0]
+    if talk.dtype != torch.float32 or talk.shape != (H, H) or not talk.is_contiguous() or H % num_kv_heads:
+        raise RuntimeError("talk_mix: talk is fp32 [H, H] contiguous, H a multiple of the key/value heads")
+    if parts.dim() != 2 or parts.stride(1) != 1 or parts.shape[1] % (H * num_kv_heads):
+        raise RuntimeError("talk_mix: parts is [T, H * G * E] with contiguous rows")
+    T, E = parts.shape[0], parts.shape[1] // (H * num_kv_heads)
+    if out is None:
+        out = torch.empty((T, H * E), dtype=parts.dtype, device=parts.device)
+    elif out.shape != (T, H * E) or out.dtype != parts.dtype or out.stride(1) != 1:
+        raise RuntimeError("talk_mix: out is [T, H * E] of the activation type")
+    check(_lib.load().semipd_talk_mix(ptr(parts), parts.stride(0), ptr(talk), ptr(out), out.stride(0), T, H, num_kv_heads, E,
+                                      dtype_code(parts.dtype), current_stream(parts.device)), "talk_mix")
+    return out
+
+
+STATE_SPACE_FUSED_DECODE_BYTES = 128 << 10     # a request's state per layer up to which a decode batch takes the one-launch form
+
+
+def state_space(proj: torch.Tensor, z_off: int, x_off: int, dt_off: int, conv_w: torch.Tensor, conv_b: Optional[torch.Tensor],
+                dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: Optional[torch.Tensor], norm_weight: torch.Tensor,
+                norm_groups: int, eps: float, state: torch.Tensor, conv_state: Optional[torch.Tensor], state_indices: torch.Tensor,
+                seq_lens: torch.Tensor, q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor], num_heads: int, groups: int,
+                state_size: int, v_dim: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The state-space recurrence behind its projection GEMM (csrc/state_space.hip).  Rows of `proj`: z [H * E] at z_off, the
+    convolution's channels x [H * E] | B [G * N] | C [G * N] at x_off, dt [H] at dt_off; conv_w [channels, taps], conv_b
+    [channels]; dt_bias / a_log / d_skip fp32 [H]; norm_weight [H * E]; state fp32 [slots, H * N * E] and conv_state fp32
+    [slots, (taps - 1) * channels] are column ranges of the requests' state rows.  Returns [T, H * E]."""
+    T, B = proj.shape[0], state_indices.shape[0]
+    inner = num_heads * v_dim
+    C = inner + 2 * groups * state_size
+    taps = conv_w.shape[1]
+    if proj.dim() != 2 or proj.stride(1) != 1:
+        raise RuntimeError("state_space: proj is 2-D with contiguous rows")
+    if conv_w.shape != (C, taps) or conv_w.dtype != proj.dtype or not conv_w.is_contiguous():
+        raise RuntimeError("state_space: conv_w is contiguous [channels, taps] of the activation type")
+    if conv_b is not None and (conv_b.shape != (C,) or conv_b.dtype != proj.dtype or not conv_b.is_contiguous()):
+        raise RuntimeError("state_space: conv_b is contiguous [channels] of the activation type")
+    for vec in (dt_bias, a_log, d_skip):
+        if vec is not None and (vec.dtype != torch.float32 or vec.shape != (num_heads,) or not vec.is_contiguous()):
+            raise RuntimeError("state_space: dt_bias / a_log / d_skip are fp32 [H]")
+    if norm_weight.shape != (inner,) or norm_weight.dtype != proj.dtype or not norm_weight.is_contiguous():
+        raise RuntimeError("state_space: norm_weight is contiguous [H * E] of the activation type")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != inner * state_size or state.stride(1) != 1:
+        raise RuntimeError("state_space: state is fp32 [slots, H * N * E]")
+    if taps > 1 and (conv_state is None or conv_state.dtype != torch.float32 or conv_state.dim() != 2
+                     or conv_state.shape[1] != (taps - 1) * C or conv_state.stride(1) != 1):
+        raise RuntimeError("state_space: conv_state is fp32 [slots, (taps - 1) * channels]")
+    if state_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64 or seq_lens.shape[0] != B:
+        raise RuntimeError("state_space: state_indices / seq_lens are int64 [B]")
+    _batch_rows("state_space", T, B, q_start, q_len)
+    if min(z_off, x_off, dt_off) < 0 or max(z_off + inner, x_off + C, dt_off + num_heads) > proj.shape[1]:
+        raise RuntimeError("state_space: a column range leaves the row")
+    if out is None:
+        out = torch.empty((T, inner), dtype=proj.dtype, device=proj.device)
+    elif out.shape != (T, inner) or out.dtype != proj.dtype or out.stride(1) != 1:
+        raise RuntimeError("state_space: out is [T, H * E] of the activation type")
+    lib = _lib.load()
+    fused = q_start is None and inner * state_size * 4 <= STATE_SPACE_FUSED_DECODE_BYTES
+    wld, work = 0, None
+    if not fused:
+        wld = int(lib.semipd_state_space_work_width(num_heads, groups, state_size, v_dim))
+        work = torch.empty((T, wld), dtype=torch.float32, device=proj.device)
+    check(lib.semipd_state_space(ptr(proj), proj.stride(0), int(z_off), int(x_off), int(dt_off), ptr(conv_w), ptr(conv_b), ptr(dt_bias),
+                                 ptr(a_log), ptr(d_skip), ptr(norm_weight), int(norm_groups), float(eps), ptr(work), wld, ptr(state),
+                                 state.stride(0), ptr(conv_state), conv_state.stride(0) if conv_state is not None else 0,
+                                 ptr(state_indices), ptr(seq_lens), ptr(q_start), ptr(q_len), B, T, num_heads, groups, state_size,
+                                 v_dim, taps, ptr(out), out.stride(0), 1 if fused else 0, dtype_code(proj.dtype),
+                                 current_stream(proj.device)), "state_space")
+    return out

@@ -116,8 +116,9 @@ def test_latent_preparation_and_store(dtype, H, D, Pr, R, rot, scaling):
         assert abs(mscale - m_ref) < 1e-12
     pool = torch.zeros(N, R + Pr, dtype=dtype, device=DEV)
     q_out = torch.zeros(T, H * (R + Pr), dtype=dtype, device=DEV)
-    ops.latent_prep(row.to(DEV), H, D, Pr, R, H * (D + Pr), nw.to(DEV), eps, pos.to(DEV), freq.to(DEV) if rot else None, rot, mscale,
-                    pool, loc.to(DEV), q_out)
+    row_d = row.to(DEV)
+    ops.latent_prep(row_d, row_d[:, H * (D + Pr): H * (D + Pr) + R + Pr], H, D, Pr, R, nw.to(DEV), eps, pos.to(DEV),
+                    freq.to(DEV) if rot else None, rot, mscale, pool, loc.to(DEV), q_out)
 
     def rotated(x, n):          # the oracle rotates positions 0 .. T-1 of one sequence: one call per token at its own position
         x = x.view(T, n, Pr)

@@ -477,7 +477,7 @@ def _penozen_kernel_pairs(s, t, window, keep, dev):
     pos = torch.arange(Tn, device=dev)
     nw = torch.ones(R, device=dev, dtype=dt)
     freq = 10000.0 ** (-2.0 * torch.arange(Pr // 2, dtype=torch.float32, device=dev) / Pr)
-    t_new = _timed(lambda: ops.latent_prep(p, H, D, Pr, R, H * (D + Pr), nw, 1e-5, pos, freq, Pr, 1.07, pool3, loc, q3))
+    t_new = _timed(lambda: ops.latent_prep(p, p[:, H * (D + Pr): H * (D + Pr) + R + Pr], H, D, Pr, R, nw, 1e-5, pos, freq, Pr, 1.07, pool3, loc, q3))
     cols = tH * tD + 2 * tG * tD + 3 * W
     tp = torch.randn(Tn, cols, device=dev, dtype=dt)
     kp3 = torch.zeros(Tn + 1, tG, tD, device=dev, dtype=dt)
