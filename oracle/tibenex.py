@@ -171,3 +171,68 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], streams: O
         if streams is not None:
             streams.append(x.clone())
     return rms_norm(x, w["final.norm"], eps) @ w["head"].float().t()
+
+
+def forward_layers(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int]):
+    """(logits, the stream after every layer)."""
+    streams: list = []
+    return forward(cfg, w, tokens, streams), streams
+
+
+def random_weights(cfg: dict, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """Random bf16 weights under the checkpoint's names, scaled so that every sublayer matters and nothing saturates."""
+    gen = torch.Generator().manual_seed(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def mat(n_out, n_in, gain=1.0):
+        return (torch.randn(n_out, n_in, generator=gen) * gain / math.sqrt(n_in)).to(torch.bfloat16)
+
+    def vec(n, scale=0.1, shift=0.0):
+        return (torch.randn(n, generator=gen) * scale + shift).to(torch.bfloat16)
+
+    w = {"embed": torch.randn(V, W, generator=gen).to(torch.bfloat16), "final.norm": vec(W, 0.1, 1.0), "head": mat(V, W)}
+    for i, layer in enumerate(cfg["layers"]):
+        pre, m = f"l{i}.", layer["mixer"]
+        w[pre + "norm1"] = vec(W, 0.1, 1.0)
+        w[pre + "ls1"] = vec(W, 0.2, 1.0)
+        w[pre + "shift"] = (torch.rand(W, generator=gen) * 0.8).to(torch.bfloat16)
+        if layer["type"] == "latent_attention":
+            H, D, P, E, R, Rq = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            w[pre + "mix.dq"] = mat(Rq, W)
+            w[pre + "mix.dq.norm"] = vec(Rq, 0.1, 1.0)
+            w[pre + "mix.uq"] = mat(H * (D + P), Rq)
+            w[pre + "mix.dkv"] = mat(R + P, W)
+            w[pre + "mix.dkv.norm"] = vec(R, 0.1, 1.0)
+            w[pre + "mix.uk"] = mat(H * D, R)
+            w[pre + "mix.uv"] = mat(H * E, R)
+            w[pre + "mix.g"] = mat(H, W)
+            w[pre + "mix.o"] = mat(W, H * E)
+        elif layer["type"] == "attention":
+            H, G, D, E = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            w[pre + "mix.q"] = mat(H * D, W)
+            w[pre + "mix.k"] = mat(G * D, W)
+            w[pre + "mix.v"] = mat(G * E, W)
+            w[pre + "mix.q.norm"] = vec(H * D, 0.2, 1.0)
+            w[pre + "mix.k.norm"] = vec(G * D, 0.2, 1.0)
+            w[pre + "mix.talk"] = (torch.eye(H) + 0.4 * torch.randn(H, H, generator=gen)).to(torch.bfloat16)
+            w[pre + "mix.temp"] = (0.5 + 1.5 * torch.rand(H, generator=gen)).to(torch.bfloat16)
+            w[pre + "mix.o"] = mat(W, H * E)
+        else:
+            H, E, N, G, n = m["heads"], m["vdim"], m["state"], m["groups"], m["conv"]
+            C = H * E + 2 * G * N
+            w[pre + "mix.in"] = mat(2 * H * E + 2 * G * N + H, W)
+            w[pre + "mix.conv"] = (torch.randn(C, n, generator=gen) * 0.5).to(torch.bfloat16)
+            w[pre + "mix.conv.b"] = vec(C, 0.2)
+            w[pre + "mix.dt_bias"] = vec(H, 0.5, -1.0)
+            w[pre + "mix.A_log"] = vec(H, 0.5, -1.0)
+            w[pre + "mix.D"] = vec(H, 0.5, 1.0)
+            w[pre + "mix.norm"] = vec(H * E, 0.1, 1.0)
+            w[pre + "mix.o"] = mat(W, H * E)
+        mlp = layer.get("mlp")
+        if mlp is not None:
+            w[pre + "norm2"] = vec(W, 0.1, 1.0)
+            w[pre + "ls2"] = vec(W, 0.2, 1.0)
+            w[pre + "mlp.gate"] = mat(mlp["ff"], W)
+            w[pre + "mlp.up"] = mat(mlp["ff"], W)
+            w[pre + "mlp.down"] = mat(W, mlp["ff"])
+    return w

@@ -153,8 +153,12 @@ class BigramEmbedding(nn.Module):
 
 
 class SiluAndMul(nn.Module):
+    def __init__(self, any_width: bool = False):
+        super().__init__()
+        self.any_width = any_width       # models whose feed-forward sizes are not bound to 16-byte rows
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.silu_and_mul(x)
+        return ops.silu_and_mul(x, any_width=self.any_width)
 
 
 # --------------------------------------------------------------------------- rotary embedding

@@ -295,7 +295,7 @@ class TibenexMLP(nn.Module):
         super().__init__()
         self.gate_up_proj = MergedColumnParallelLinear(hidden_size, [ff, ff], params_dtype=dtype)
         self.down_proj = RowParallelLinear(ff, hidden_size, params_dtype=dtype)
-        self.act_fn = SiluAndMul()
+        self.act_fn = SiluAndMul(any_width=True)
 
     def forward(self, x):
         return self.down_proj(gate_up_silu(x, self.gate_up_proj, self.act_fn))

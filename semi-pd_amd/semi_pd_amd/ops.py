@@ -67,8 +67,10 @@ def fused_add_rmsnorm(input: torch.Tensor, residual: torch.Tensor, weight: torch
 
 
 # --------------------------------------------------------------------------- activation
-def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    if input.shape[-1] * input.dtype.itemsize % 16 != 0:
+def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None, any_width: bool = False) -> torch.Tensor:
+    """any_width: rows that are no multiple of 16 bytes are taken too (the kernel's element-wise form) instead of refused like
+    the reference's op refuses them."""
+    if not any_width and input.shape[-1] * input.dtype.itemsize % 16 != 0:
         raise ValueError("The pointers must be multiple of 16 bytes.")
     d = input.shape[-1] // 2
     if out is not None:
