@@ -495,9 +495,9 @@ def main():
     ap.add_argument("--arch-compare", action="store_true",
                     help="instead of the serving line: Kudirax next to Llama at equal layer sizes, models and kernels "
                          "(tools/arch_compare.py); one JSON object of its own")
-    ap.add_argument("--arch-design", default="kudirax", choices=["kudirax", "tigotar", "penozen"],
+    ap.add_argument("--arch-design", default="kudirax", choices=["kudirax", "tigotar", "penozen", "tibenex"],
                     help="--arch-compare: which design is measured (kudirax: next to Llama; tigotar: next to Kudirax; penozen: next "
-                         "to Tigotar)")
+                         "to Tigotar; tibenex: next to Penozen)")
     ap.add_argument("--arch-sizes", default="", help="--arch-compare: comma-separated size names (default: all)")
     ap.add_argument("--arch-chunk", type=int, default=1024, help="--arch-compare: positions per attention block (0: none)")
     args = ap.parse_args()

@@ -39,7 +39,7 @@ from semi_pd_amd.distributed import get_tensor_model_parallel_world_size
 from semi_pd_amd.layers.attention_backend import RadixAttention
 from semi_pd_amd.layers.basic import (LogitsProcessor, MergedColumnParallelLinear, ParallelLMHead, RowParallelLinear, SiluAndMul,
                                       VocabParallelEmbedding, dense_linear, gate_up_silu)
-from semi_pd_amd.models.penozen import stretched_frequencies
+from semi_pd_amd.models.penozen import EXPAND_MIN_TOKENS, context_rows, stretched_frequencies
 
 
 @dataclass
@@ -162,13 +162,16 @@ class TibenexConfig:
 
 def tibenex_uniform(vocab_size: int, hidden_size: int, pattern: str, ff: int, heads: int, kv_heads: int, dim: int, vdim: int,
                     rot_dim: int, kv_rank: int, q_rank: int, ssm_heads: int, ssm_vdim: int, state: int, groups: int,
-                    norm_groups: int = 1, conv: int = 4, alpha: float = 2.0, norm_eps: float = 1e-6) -> TibenexConfig:
-    """A configuration from a pattern of layer kinds: 'l' latent attention, 'a' attention, 'm' state space (benchmarks, tests)."""
+                    norm_groups: int = 1, conv: int = 4, alpha: float = 2.0, norm_eps: float = 1e-6, latent_heads: int = 0,
+                    latent_dim: int = 0, latent_vdim: int = 0) -> TibenexConfig:
+    """A configuration from a pattern of layer kinds: 'l' latent attention (latent_heads / latent_dim / latent_vdim, by default
+    the attention layers' sizes), 'a' attention, 'm' state space (benchmarks, tests)."""
+    lh, ld, lv = latent_heads or heads, latent_dim or dim, latent_vdim or vdim
     layers = []
     for ch in pattern:
         if ch == "l":
             layers.append(TibenexLayerConfig("latent_attention", TibenexLatentConfig(
-                heads, dim, rot_dim, vdim, kv_rank, q_rank, (dim + rot_dim) ** -0.5, RotationConfig(rot_dim, 10000.0)), ff))
+                lh, ld, rot_dim, lv, kv_rank, q_rank, (ld + rot_dim) ** -0.5, RotationConfig(rot_dim, 10000.0)), ff))
         elif ch == "a":
             layers.append(TibenexLayerConfig("attention", TibenexAttentionConfig(
                 heads, kv_heads, dim, vdim, dim ** -0.5, RotationConfig(dim, 10000.0)), ff))
@@ -203,6 +206,49 @@ class TibenexLatentAttention(nn.Module):
         self.register_buffer("freq", freq, persistent=False)
         # the pool row [latent | rotated key part] is the one key/value head of every query head; its first R elements the value
         self.attn = RadixAttention(H, R + P, mc.scale, 1, region, v_head_dim=R)
+        # prompt batches: keys [W_uk,h c | r] of all heads from the latent rows in one GEMM, W = [[W_uk,h, 0], [0, I]] per head
+        self.register_buffer("w_key_rows", torch.empty(0, dtype=dtype), persistent=False)
+        self.register_buffer("w_val_rows", torch.empty(0, dtype=dtype), persistent=False)     # [W_uv | 0]: values from the same rows
+
+    def post_load_weights(self):
+        mc = self.mc
+        H, D, P, R = mc.heads, mc.dim, mc.rot_dim, mc.kv_rank
+        w = torch.zeros(H, D + P, R + P, dtype=self.w_uk.dtype, device=self.w_uk.device)
+        w[:, :D, :R] = self.w_uk
+        w[:, D:, R:] = torch.eye(P, dtype=w.dtype, device=w.device)
+        self.w_key_rows = w.view(H * (D + P), R + P)
+        wv = torch.zeros(H * mc.vdim, R + P, dtype=self.w_uv.dtype, device=self.w_uv.device)
+        wv[:, :R] = self.w_uv.view(H * mc.vdim, R)
+        self.w_val_rows = wv
+
+    def expands_keys(self, forward_batch) -> bool:
+        """Whether a batch expands the keys and values of its requests' tokens from the latent rows and attends head by head
+        (fewer multiply-adds per query-key pair: D + P + E against 2 R + P) instead of attending over the latent rows: prompt
+        batches whose context is not much longer than their new tokens.  SEMIPD_LATENT_EXPAND: 0 never, 2 every extend batch."""
+        knob = os.environ.get("SEMIPD_LATENT_EXPAND", "1")
+        if knob == "0" or not forward_batch.forward_mode.is_extend() or self.w_key_rows.numel() == 0:
+            return False
+        new = forward_batch.extend_num_tokens
+        ctx = new + sum(forward_batch.extend_prefix_lens_cpu)
+        return knob == "2" or (new >= EXPAND_MIN_TOKENS and ctx <= 4 * new)
+
+    def _forward_expanded(self, p: torch.Tensor, q: torch.Tensor, forward_batch) -> torch.Tensor:
+        mc = self.mc
+        H, D, P, E, R = mc.heads, mc.dim, mc.rot_dim, mc.vdim, mc.kv_rank
+        T = p.shape[0]
+        pool = forward_batch.token_to_kv_pool.get_key_buffer(self.attn.layer_id)
+        pool = pool.view(pool.shape[0], -1)
+        ops.latent_prep(q, p[:, mc.q_rank: mc.q_rank + self.c_size], H, D, P, R, self.latent_norm, self.eps, forward_batch.positions,
+                        self.freq if mc.rot.dims else None, mc.rot.dims, self.mscale, pool, forward_batch.out_cache_loc, halves=True)
+        slots, table, rows = context_rows(forward_batch)
+        ctx = ops.gather_rows(pool, slots)                                    # [N, R + P]: every request's tokens, in order
+        keys = dense_linear(ctx, self.w_key_rows)                             # [N, H * (D + P)]
+        vals = dense_linear(ctx, self.w_val_rows)                             # [N, H * E]
+        out = torch.empty((T, H * E), dtype=p.dtype, device=p.device)
+        ops.local_attention_fwd(q, out, keys.view(-1, H, D + P), vals.view(-1, H, E), table, rows, forward_batch.seq_lens,
+                                forward_batch.extend_start_loc, forward_batch.extend_seq_lens, max(forward_batch.extend_seq_lens_cpu),
+                                mc.scale, 0.0, 0, None, None, form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")))
+        return self.out_proj(ops.sigmoid_gate_heads_(out, p[:, mc.q_rank + self.c_size:]))
 
     def forward(self, h: torch.Tensor, forward_batch) -> torch.Tensor:
         mc = self.mc
@@ -211,6 +257,8 @@ class TibenexLatentAttention(nn.Module):
         p = self.in_proj(h)
         cq = ops.rmsnorm(p[:, : mc.q_rank], self.q_norm, self.eps)
         q = dense_linear(cq, self.q_up)                                            # [T, H * (D + P)]
+        if self.expands_keys(forward_batch):
+            return self._forward_expanded(p, q, forward_batch)
         pool = forward_batch.token_to_kv_pool.get_key_buffer(self.attn.layer_id)
         q_in = torch.empty((T, H * (R + P)), dtype=p.dtype, device=p.device)
         ops.latent_prep(q, p[:, mc.q_rank: mc.q_rank + self.c_size], H, D, P, R, self.latent_norm, self.eps, forward_batch.positions,
@@ -401,7 +449,9 @@ class TibenexForCausalLM(nn.Module):
             p.requires_grad_(False)
 
     def post_load_weights(self):
-        pass
+        for layer in self.layers:
+            if isinstance(layer.mix, TibenexLatentAttention):
+                layer.mix.post_load_weights()
 
     @property
     def kv_geometry(self):

@@ -546,6 +546,23 @@ def test_eager_decode_steps_with_the_separate_shift_launch(dtype, tmp_path, monk
         assert _rel_err(got[n], O.forward(cfg, w, prompts[n]), dtype != "float32") < LIMIT[dtype], n
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mixed", "awkward", "attention_only"])
+def test_prompt_batches_that_expand_keys_from_the_latent_rows(name, dtype, tmp_path, monkeypatch):
+    """Every extend batch takes the form that large prompt batches take by themselves: keys and values of all heads expanded
+    from the requests' latent rows (those of earlier portions included), attention head by head, the heads' gates behind
+    it.  Decode steps between the portions attend over the latent rows; both forms have to agree with the plain model."""
+    monkeypatch.setenv("SEMIPD_LATENT_EXPAND", "2")
+    cfg = CONFIGS[name]
+    w = _write_checkpoint(str(tmp_path), cfg, seed=7)
+    sched = _scheduler(str(tmp_path), dtype, max_tokens=336)
+    prompts = {"x": _tokens(120, cfg["vocab"], 3), "y": _tokens(45, cfg["vocab"], 4), "z": _tokens(70, cfg["vocab"], 5)}
+    got = _run_schedule(sched, prompts, [[("x", 64), ("y", 2)], [("x", 1), ("y", 1)], [("x", 2), ("y", 40), ("z", 33)], [("x", 1), ("z", 1)],
+                                         [("x", 52), ("y", 2), ("z", 36)]])
+    for n in prompts:
+        assert _rel_err(got[n], O.forward(cfg, w, prompts[n]), dtype != "float32") < LIMIT[dtype], n
+
+
 def test_a_far_token_decides_the_logits(tmp_path):
     """Weights made so that attention's first head looks far back: the temperature of one head of the talking attention is
     large, so its softmax is nearly one-hot on some key hundreds of tokens back; replacing that far token has to change the

@@ -2,7 +2,9 @@
 with `--arch-design tigotar`: Tigotar next to Kudirax, the closest model of the framework (fp32 stream, norms on the
 sublayers' outputs, attention over a bounded range of keys through the same kernel family), at equal layer sizes;
 with `--arch-design penozen`: Penozen next to Tigotar (fp32 stream, attention and a recurrence over pooled state rows,
-a mixture of experts behind them).
+a mixture of experts behind them);
+with `--arch-design tibenex`: Tibenex next to Penozen (fp32 stream, latent attention, a recurrence with a matrix state and a
+short convolution over pooled state rows).
 
 Two parts, printed as one JSON object:
   * "models": prefill and decode throughput of a few-layer model of each design at layer sizes of real models, both driven
@@ -567,7 +569,200 @@ def main_penozen(args) -> dict:
     return result
 
 
+TIBENEX_SIZES = {
+    # latent attention as in PENOZEN_SIZES (+ a query latent of `qrank`); attention whose heads talk: `theads` queries over `tkv`
+    # key/value heads of `tdim` / `tvdim` (value row = tkv * tvdim elements); state space: `sheads` heads of `svdim` values,
+    # `state` rows per head, `groups` groups; a dense gated feed-forward of `ff`
+    "8b-layer": dict(hidden=4096, heads=32, dim=64, rot=64, vdim=128, rank=192, qrank=1536, theads=32, tkv=2, tdim=128, tvdim=128,
+                     sheads=128, svdim=64, state=128, groups=8, ff=14336, vocab=32000),
+    "3b-layer": dict(hidden=3072, heads=24, dim=64, rot=64, vdim=128, rank=192, qrank=1024, theads=24, tkv=2, tdim=128, tvdim=128,
+                     sheads=96, svdim=64, state=128, groups=8, ff=8192, vocab=32000),
+    "1b-layer": dict(hidden=2048, heads=32, dim=32, rot=32, vdim=64, rank=96, qrank=768, theads=32, tkv=4, tdim=64, tvdim=64,
+                     sheads=64, svdim=64, state=64, groups=8, ff=8192, vocab=32000),
+}
+
+
+def _tibenex_kernel_pairs(s, pz, dev):
+    """[(what, Tibenex kernel's record, like kernel's record)]: `s` Tibenex's layer shape, `pz` Penozen's at the same size."""
+    from semi_pd_amd import ops
+    dt = torch.bfloat16
+    W = s["hidden"]
+    out = []
+
+    def rec(tm, nbytes=0.0, flops=0.0, vflops=0.0):
+        frac = max(nbytes / tm / HBM, flops / tm / MFMA, vflops / tm / VALU)
+        return {"us": round(tm * 1e6, 1), "TB_per_s": round(nbytes / tm / 1e12, 2),
+                "TFLOP_per_s": round(max(flops, vflops) / tm / 1e12, 1), "of_roofline": round(frac, 3)}
+
+    B, L = 4, 2048
+    T = B * L
+    B2, C = 32, 2000
+    rows, lens = torch.arange(B, device=dev), torch.full((B,), L, device=dev, dtype=torch.int64)
+    q_start = torch.arange(B, device=dev, dtype=torch.int32) * L
+    q_len = torch.full((B,), L, device=dev, dtype=torch.int32)
+    rows2, lens2 = torch.arange(B2, device=dev), torch.full((B2,), C, device=dev, dtype=torch.int64)
+    r2t = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(B, L).contiguous()
+    r2t2 = (torch.arange(B2 * C, device=dev, dtype=torch.int32) + 1).view(B2, C).contiguous()
+    # ---- the seam: norm after the sum (+ the shift for the next mixer in decode batches) against stream += y, norm -----------
+    st_slab = torch.zeros(B2 + 1, W, device=dev)
+    st32 = torch.arange(1, B2 + 1, device=dev)
+    for Tn in (8192, 32):
+        y = torch.randn(Tn, W, device=dev, dtype=dt)
+        res = torch.randn(Tn, W, device=dev, dtype=torch.float32)
+        w = torch.ones(W, device=dev, dtype=dt)
+        if Tn > 32:
+            t_new = _timed(lambda: ops.postnorm_stream(y, w, res, 2.0, w, 1e-6))
+            nb_new = Tn * W * (2 + 4 + 4 + 2.0)
+            what = "stream = norm(alpha stream + scale * y), copy for the next sublayer"
+        else:
+            t_new = _timed(lambda: ops.postnorm_stream(y, w, res, 2.0, w, 1e-6, shift_mu=w, prev=st_slab, state_indices=st32, seq_lens=lens2))
+            nb_new = Tn * W * (2 + 4 + 4 + 2.0 + 8)
+            what = "stream = norm(alpha stream + scale * y), the next mixer's shifted input, the previous row in the state"
+        t_old = _timed(lambda: ops.rms_stream(y, res, w, 1e-5, 1.0))
+        out.append((f"{what}, {Tn} rows of {W} (like: stream += y, next input = RMS norm(stream))",
+                    rec(t_new, nbytes=nb_new), rec(t_old, nbytes=Tn * W * (2 + 4 + 4 + 2.0))))
+    res = torch.randn(T, W, device=dev, dtype=torch.float32)
+    mu = torch.rand(W, device=dev).to(dt)
+    st4 = torch.arange(1, B + 1, device=dev)
+    t_new = _timed(lambda: ops.token_shift(res, mu, st_slab, st4, lens, q_start, q_len))
+    t_old = _timed(lambda: ops.rms_stream(None, res, mu, 1e-5, 1.0))
+    out.append((f"token shift of a prompt batch, {T} rows of {W} (reads two fp32 rows per row; like: RMS norm of the stream into the "
+                "activation type, one row per row)", rec(t_new, nbytes=T * W * (4 + 4 + 2.0)), rec(t_old, nbytes=T * W * (4 + 2.0))))
+    # ---- attention whose heads talk ----------------------------------------------------------------------------------------
+    H, G, D, E = s["theads"], s["tkv"], s["tdim"], s["tvdim"]
+    pH, pD, pP, pE, pR = pz["heads"], pz["dim"], pz["rot"], pz["vdim"], pz["rank"]
+    Tn = 8192
+    p = torch.randn(Tn, (H + G) * D + G * E, device=dev, dtype=dt)
+    kp = torch.zeros(max(Tn, B2 * C) + 1, G, D, device=dev, dtype=dt)
+    vp = torch.zeros(max(Tn, B2 * C) + 1, G, E, device=dev, dtype=dt)
+    loc, pos = torch.arange(1, Tn + 1, device=dev), torch.arange(Tn, device=dev)
+    qw, kw = torch.ones(H * D, device=dev, dtype=dt), torch.ones(G * D, device=dev, dtype=dt)
+    temp = torch.ones(H, device=dev)
+    freq = 10000.0 ** (-2.0 * torch.arange(D // 2, dtype=torch.float32, device=dev) / D)
+    t_new = _timed(lambda: ops.qk_norm_rope_kv_store(p, H, G, D, E, H * D, (H + G) * D, qw, kw, 1e-6, pos, freq, D, False, 1.0, temp, kp, vp, loc))
+    pp = torch.randn(Tn, pH * (pD + pP) + pR + pP + pH * pE, device=dev, dtype=dt)
+    pool3 = torch.zeros(Tn + 1, pR + pP, device=dev, dtype=dt)
+    q3 = torch.empty(Tn, pH * (pR + pP), device=dev, dtype=dt)
+    nw = torch.ones(pR, device=dev, dtype=dt)
+    pfreq = 10000.0 ** (-2.0 * torch.arange(pP // 2, dtype=torch.float32, device=dev) / pP)
+    t_old = _timed(lambda: ops.latent_prep(pp, pp[:, pH * (pD + pP): pH * (pD + pP) + pR + pP], pH, pD, pP, pR, nw, 1e-5, pos, pfreq, pP, 1.07,
+                                           pool3, loc, q3))
+    out.append((f"norm of q and k over the whole projection + rotation + temperature + KV store, {Tn} tokens, {H} / {G} heads of {D} / {E} "
+                "(like: latent norm, rotation of the shared key part and the heads' rotated query parts, pool store)",
+                rec(t_new, nbytes=Tn * 2.0 * (2 * H * D + 2 * G * D + 2 * G * E)), rec(t_old, nbytes=Tn * 2.0 * (2 * (pR + pP) + 2 * pH * pP))))
+    kp.normal_()
+    vp.normal_()
+    q = torch.randn(T, H * D, device=dev, dtype=dt)
+    parts = torch.empty(T, H * G * E, device=dev, dtype=dt)
+    talk = torch.eye(H, device=dev) + 0.1
+    o = torch.empty(T, H * E, device=dev, dtype=dt)
+
+    def talking():
+        ops.shared_value_attention_fwd(q, parts, kp, vp, r2t, rows, lens, q_start, q_len, L, D ** -0.5)
+        ops.talk_mix(parts, talk, G, out=o)
+
+    t_new = _timed(talking)
+    pairs = B * L * (L + 1) / 2
+    # the like kernel: Penozen's prompt attention head by head over expanded keys and values, with the sink and the gate
+    keys = torch.randn(T, pH, pD + pP, device=dev, dtype=dt)
+    vals = torch.randn(T, pH, pE, device=dev, dtype=dt)
+    tab = torch.arange(T, device=dev, dtype=torch.int32).view(B, L).contiguous()
+    qh = torch.randn(T, pH * (pD + pP), device=dev, dtype=dt)
+    oh = torch.empty(T, pH * pE, device=dev, dtype=dt)
+    gate = torch.randn(T, pH * pE, device=dev, dtype=dt)
+    sink = torch.zeros(pH, device=dev)
+    t_old = _timed(lambda: ops.local_attention_fwd(qh, oh, keys, vals, tab, rows, lens, q_start, q_len, L, 0.1, 0.0, 0, sink, gate))
+    out.append((f"prompt attention, {B} x {L} tokens, {H} heads of {D} whose weights meet the values of all {G} key/value heads of {E}, + the "
+                f"mix of the heads ({H} x {H}) (like: {pH} heads of {pD + pP} / {pE}, causal softmax with a sink and the output gate)",
+                rec(t_new, flops=2.0 * H * (D + G * E) * pairs + 2.0 * T * H * H * E), rec(t_old, flops=2.0 * pH * (pD + pP + pE) * pairs)))
+    q2 = torch.randn(B2, H * D, device=dev, dtype=dt)
+    parts2 = torch.empty(B2, H * G * E, device=dev, dtype=dt)
+    o2 = torch.empty(B2, H * E, device=dev, dtype=dt)
+
+    def talking_decode():
+        ops.shared_value_attention_fwd(q2, parts2, kp, vp, r2t2, rows2, lens2, None, None, 1, D ** -0.5)
+        ops.talk_mix(parts2, talk, G, out=o2)
+
+    t_new = _timed(talking_decode)
+    pool2 = torch.randn(B2 * C + 1, pR + pP, device=dev, dtype=dt)
+    ql = torch.randn(B2, pH * (pR + pP), device=dev, dtype=dt)
+    ol = torch.empty(B2, pH * pR, device=dev, dtype=dt)
+    splits = max(1, min(16, 512 // (B2 * ((pH + 15) // 16)), C // 128))
+    t_old = _timed(lambda: ops.latent_attention_fwd(ql, ol, pool2, pR, r2t2, rows2, lens2, None, None, 1, 0.1, sink, n_splits=splits))
+    out.append((f"decode attention, {B2} requests at {C} tokens, {G} key/value heads of {D} / {E}, + the mix of the heads (like: every latent "
+                f"row of {pR} + {pP} once for all {pH} heads, {splits} workgroups share a request's keys, + merge)",
+                rec(t_new, nbytes=B2 * G * (D + E) * 2.0 * C), rec(t_old, nbytes=B2 * (pR + pP) * 2.0 * C)))
+    # ---- the recurrences: a prompt batch and a decode batch ----------------------------------------------------------------
+    SH, SE, N, SG, taps = s["sheads"], s["svdim"], s["state"], s["groups"], 4
+    inner, Cc = SH * SE, SH * SE + 2 * SG * N
+    width = 2 * inner + 2 * SG * N + SH
+    conv_w = torch.randn(Cc, taps, device=dev, dtype=dt) * 0.5
+    conv_b = torch.zeros(Cc, device=dev, dtype=dt)
+    a_log, dt_bias, dsk = torch.zeros(SH, device=dev) - 1.0, torch.zeros(SH, device=dev), torch.ones(SH, device=dev)
+    onw = torch.ones(inner, device=dev, dtype=dt)
+    S = torch.zeros(B2 + 1, inner * N, device=dev)
+    cs = torch.zeros(B2 + 1, (taps - 1) * Cc, device=dev)
+    sp = torch.randn(T, width, device=dev, dtype=dt)
+    t_new = _timed(lambda: ops.state_space(sp, 0, inner, inner + Cc, conv_w, conv_b, dt_bias, a_log, dsk, onw, 1, 1e-5, S, cs, st4, lens,
+                                           q_start, q_len, SH, SG, N, SE), iters=5, warm=1)
+    DH, DG, KD, VD = pz["dheads"], pz["kv"], pz["kdim"], pz["dvdim"]
+    gd, hv = DG * KD, DH * VD
+    dwidth = 2 * gd + 2 * hv + 2 * DH
+    offs = [0, gd, 2 * gd, 2 * gd + hv, 2 * gd + 2 * hv, 2 * gd + 2 * hv + DH]
+    cw = [torch.randn(n, taps, device=dev, dtype=dt) * 0.5 for n in (gd, gd, hv)]
+    da_log, ddt = torch.zeros(DH, device=dev) - 1.0, torch.zeros(DH, device=dev)
+    dnw = torch.ones(VD, device=dev, dtype=dt)
+    dS = torch.zeros(B2 + 1, DH * KD * VD, device=dev)
+    dcs = torch.zeros(B2 + 1, (taps - 1) * (2 * gd + hv), device=dev)
+    dp = torch.randn(T, dwidth, device=dev, dtype=dt)
+    t_old = _timed(lambda: ops.delta_rule(dp, offs, cw[0], cw[1], cw[2], da_log, ddt, dnw, 1e-5, dS, dcs, st4, lens, q_start, q_len, DH, DG,
+                                          KD, VD), iters=5, warm=1)
+    out.append((f"state-space recurrence over {B} x {L} tokens, {SH} heads of {N} x {SE} in {SG} groups (convolution, step sizes, the "
+                f"recurrence, gate and grouped norm; 4 flop per element of S and token on the vector units; like: gated delta rule, {DH} "
+                f"heads of {KD} x {VD}, 8 flop per element)",
+                rec(t_new, nbytes=T * 2.0 * (width + inner), vflops=4.0 * T * inner * N),
+                rec(t_old, nbytes=T * 2.0 * (dwidth + hv), vflops=8.0 * T * DH * KD * VD)))
+    spd = torch.randn(B2, width, device=dev, dtype=dt)
+    t_new = _timed(lambda: ops.state_space(spd, 0, inner, inner + Cc, conv_w, conv_b, dt_bias, a_log, dsk, onw, 1, 1e-5, S, cs, st32, lens2,
+                                           None, None, SH, SG, N, SE))
+    dpd = torch.randn(B2, dwidth, device=dev, dtype=dt)
+    t_old = _timed(lambda: ops.delta_rule(dpd, offs, cw[0], cw[1], cw[2], da_log, ddt, dnw, 1e-5, dS, dcs, st32, lens2, None, None, DH, DG,
+                                          KD, VD))
+    out.append((f"state-space decode step, {B2} requests (reads and writes {inner * N * 4 / 1e6:.1f} MB of state per request; like: gated "
+                f"delta rule decode step, {DH * KD * VD * 4 / 1e6:.1f} MB per request)",
+                rec(t_new, nbytes=B2 * inner * N * 4.0 * 2), rec(t_old, nbytes=B2 * DH * KD * VD * 4.0 * 2)))
+    return out
+
+
+def main_tibenex(args) -> dict:
+    from semi_pd_amd.models.penozen import penozen_uniform
+    from semi_pd_amd.models.tibenex import tibenex_uniform
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    names = [n for n in (getattr(args, "arch_sizes", "") or ",".join(TIBENEX_SIZES)).split(",") if n]
+    result = {"what": "Tibenex next to Penozen at equal layer sizes", "dtype": "bf16", "data": "synthetic", "models": {}, "kernels": {}}
+    for name in names:
+        s, pz = TIBENEX_SIZES[name], PENOZEN_SIZES[name]
+        result["kernels"][name] = [
+            {"kernel": what, "tibenex": new, "like": old,
+             "roofline_fraction_ratio": round(new["of_roofline"] / max(old["of_roofline"], 1e-9), 2)}
+            for what, new, old in _tibenex_kernel_pairs(s, pz, dev)]
+        tcfg = tibenex_uniform(s["vocab"], s["hidden"], "lmam", s["ff"], s["theads"], s["tkv"], s["tdim"], s["tvdim"], s["rot"], s["rank"],
+                               s["qrank"], s["sheads"], s["svdim"], s["state"], s["groups"], latent_heads=s["heads"], latent_dim=s["dim"],
+                               latent_vdim=s["vdim"])
+        pcfg = penozen_uniform(pz["vocab"], pz["hidden"], "adad", pz["heads"], pz["dim"], pz["rot"], pz["vdim"], pz["rank"], pz["dheads"],
+                               pz["kv"], pz["kdim"], pz["dvdim"], pz["experts"], pz["top"], pz["ff"] // pz["top"])
+        result["models"][name] = {
+            "layers": 4,
+            "tibenex": _model_throughput(tcfg, 2048, 4, 32, 1100, 20),
+            "penozen": _model_throughput(pcfg, 2048, 4, 32, 1100, 20)}
+    print(json.dumps(result), flush=True)
+    return result
+
+
 def main(args) -> dict:
+    if getattr(args, "arch_design", "kudirax") == "tibenex":
+        return main_tibenex(args)
     if getattr(args, "arch_design", "kudirax") == "tigotar":
         return main_tigotar(args)
     if getattr(args, "arch_design", "kudirax") == "penozen":
