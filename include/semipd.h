@@ -970,12 +970,13 @@ int semipd_qk_norm_rope_kv_store(void* qkv, int64_t ld, int64_t num_tokens, int 
                                  const int64_t* positions, const float* freq, int rot_dims, int halves, float mscale,
                                  const float* head_scale, void* k_pool, void* v_pool, const int64_t* loc, int dtype, void* stream);
 /* semipd_local_attention (causal, softmax) whose value row of a slot is ONE head of v_row elements read by the queries of
- * every key/value head: out [T, heads * v_row]. */
+ * every key/value head: out [T, heads * v_row].  n_splits / partial as in semipd_latent_attention (partial fp32
+ * [rows, heads, n_splits, v_row + 2]). */
 int semipd_shared_value_attention(const void* q, int64_t q_ld, void* out, int64_t out_ld, const void* k_pool, const void* v_pool,
                                   const int32_t* req_to_token, int64_t req_to_token_stride, const int64_t* req_pool_indices,
                                   const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len, int64_t batch,
                                   int64_t num_tokens, int64_t max_q_len, int num_q_heads, int num_kv_heads, int qk_dim, int v_row,
-                                  float scale, int form, int dtype, void* stream);
+                                  float scale, int n_splits, float* partial, int form, int dtype, void* stream);
 /* out[t, h, :] = sum_g talk[h, g] * parts[t, g, c(h), :], parts [T, heads, kv heads, v_dim], c(h) the key/value head of h. */
 int semipd_talk_mix(const void* parts, int64_t parts_ld, const float* talk, void* out, int64_t out_ld, int64_t num_tokens,
                     int num_q_heads, int num_kv_heads, int v_dim, int dtype, void* stream);

@@ -418,18 +418,44 @@ __global__ void __launch_bounds__(256) qk_norm_rope_kv_store_kernel(T* __restric
 // the values of its own key/value head c(h).  The sum over the keys is linear, so
 //     out_h = sum_g talk[h, g] * (w_g applied to the values of head c(h)),
 // and `parts` [T, H, G, E] holds w_g applied to the values of EVERY key/value head (attention whose value row is shared).
-// A workgroup per token, a thread per element of out [T, H * E]; fp32 sums.
-template <typename T>
+// A workgroup per token, a thread per element of out [T, H * E]; fp32 sums.  STAGED: the token's row of `parts` and the mix
+// matrix go through LDS first (every element of the row is read by the H / G heads of its key/value head).
+template <typename T, bool STAGED>
 __global__ void __launch_bounds__(256) talk_mix_kernel(const T* __restrict__ parts, int64_t p_ld, const float* __restrict__ talk,
                                                        T* __restrict__ out, int64_t out_ld, int H, int G, int E) {
+  extern __shared__ float mix_l[];         // STAGED: talk [H * H] | the row [H * G * E]
   const int64_t t = blockIdx.x;
   const T* p = parts + t * p_ld;
   const int per = H / G;
-  for (int i = threadIdx.x; i < H * E; i += 256) {
-    const int h = i / E, e = i - h * E, c = h / per;
-    float y = 0.f;
-    for (int g = 0; g < H; ++g) y += talk[h * H + g] * Elem<T>::to_f(p[((int64_t)g * G + c) * E + e]);
-    out[t * out_ld + i] = Elem<T>::from_f(y);
+  if constexpr (STAGED) {
+    float* tk = mix_l;
+    float* pr = mix_l + H * H;
+    for (int i = threadIdx.x; i < H * H; i += 256) tk[i] = talk[i];
+    const int n = H * G * E;
+    constexpr int V = Elem<T>::kVec;
+    if (n % V == 0 && p_ld % V == 0 && (reinterpret_cast<uintptr_t>(parts) & 15u) == 0) {
+      for (int i = threadIdx.x * V; i < n; i += 256 * V) {
+        const Vec16<T> v = load16(p + i);
+#pragma unroll
+        for (int u = 0; u < V; ++u) pr[i + u] = Elem<T>::to_f(v.e[u]);
+      }
+    } else {
+      for (int i = threadIdx.x; i < n; i += 256) pr[i] = Elem<T>::to_f(p[i]);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < H * E; i += 256) {
+      const int h = i / E, e = i - h * E, c = h / per;
+      float y = 0.f;
+      for (int g = 0; g < H; ++g) y += tk[h * H + g] * pr[(g * G + c) * E + e];
+      out[t * out_ld + i] = Elem<T>::from_f(y);
+    }
+  } else {
+    for (int i = threadIdx.x; i < H * E; i += 256) {
+      const int h = i / E, e = i - h * E, c = h / per;
+      float y = 0.f;
+      for (int g = 0; g < H; ++g) y += talk[h * H + g] * Elem<T>::to_f(p[((int64_t)g * G + c) * E + e]);
+      out[t * out_ld + i] = Elem<T>::from_f(y);
+    }
   }
 }
 
@@ -1407,11 +1433,13 @@ extern "C" int semipd_shared_value_attention(const void* q, int64_t q_ld, void* 
                                              const void* v_pool, const int32_t* req_to_token, int64_t req_to_token_stride,
                                              const int64_t* req_pool_indices, const int64_t* seq_lens, const int32_t* q_start,
                                              const int32_t* q_len, int64_t batch, int64_t num_tokens, int64_t max_q_len,
-                                             int num_q_heads, int num_kv_heads, int qk_dim, int v_row, float scale, int form,
-                                             int dtype, void* stream) {
+                                             int num_q_heads, int num_kv_heads, int qk_dim, int v_row, float scale, int n_splits,
+                                             float* partial, int form, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(n_splits >= 0 && n_splits <= 64 && (n_splits <= 1 || partial != nullptr), SEMIPD_EINVAL,
+                   "shared_value_attention: up to 64 slices of the keys, with room for their partial sums");
   LocalAttnArgs a{q, q_ld, nullptr, 0, out, out_ld, k_pool, v_pool, req_to_token, req_to_token_stride, req_pool_indices,
                   seq_lens, q_start, q_len, batch, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_row, nullptr, scale, 0.f,
-                  0, 0, 0, 0, nullptr, 0, 1.0f, 0, 0, 0, nullptr, 1};
+                  0, 0, 0, 0, nullptr, 0, 1.0f, 0, 0, n_splits, partial, 1};
   return launch_local_attention(a, max_q_len, form, dtype, stream);
 }
 
@@ -1423,8 +1451,14 @@ extern "C" int semipd_talk_mix(const void* parts, int64_t parts_ld, const float*
   SEMIPD_CHECK_ARG(parts && talk && out && parts_ld >= (int64_t)num_q_heads * num_kv_heads * v_dim &&
                        out_ld >= (int64_t)num_q_heads * v_dim,
                    SEMIPD_EINVAL, "talk_mix: null pointer or rows too short");
-  SEMIPD_DISPATCH_DTYPE(dtype, T,
-                        hipLaunchKernelGGL((talk_mix_kernel<T>), dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream),
-                                           (const T*)parts, parts_ld, talk, (T*)out, out_ld, num_q_heads, num_kv_heads, v_dim));
+  const size_t staged = ((size_t)num_q_heads * num_q_heads + (size_t)num_q_heads * num_kv_heads * v_dim) * sizeof(float);
+  SEMIPD_DISPATCH_DTYPE(dtype, T, {
+    if (staged <= 65536)
+      hipLaunchKernelGGL((talk_mix_kernel<T, true>), dim3((unsigned)num_tokens), dim3(256), staged, as_stream(stream),
+                         (const T*)parts, parts_ld, talk, (T*)out, out_ld, num_q_heads, num_kv_heads, v_dim);
+    else
+      hipLaunchKernelGGL((talk_mix_kernel<T, false>), dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream),
+                         (const T*)parts, parts_ld, talk, (T*)out, out_ld, num_q_heads, num_kv_heads, v_dim);
+  });
   return launch_status("talk_mix");
 }

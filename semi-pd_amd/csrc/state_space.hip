@@ -8,16 +8,17 @@
 // then y * silu(z), an RMS norm over each of `norm_groups` equal parts of the row, times a weight.  Everything behind the
 // projection GEMM is fp32 whatever the activation type.
 //
-//  * ssm_prep_kernel: a workgroup per token: convolution + bias + silu of the token's x | B | C channels (inputs in front
+//  * ssm_prep_kernel: a workgroup per (token, 1024 channels), four channels per thread where alignment allows: convolution + bias + silu of the token's x | B | C channels (inputs in front
 //    of the portion come from the state row), dt and the decay -> an fp32 work row per token.
 //  * ssm_conv_state_kernel: the last taps - 1 inputs of the portion (shifted in behind what the row held) -> state row.
 //  * ssm_scan_kernel: ONE WAVE per (request, head, block of 64 / NS columns of S); a column of S lives in the registers of NS
 //    adjacent lanes, NPT rows each, so a step is one multiply-add per register for the update, one for the read-out, and a
-//    log2(NS)-step lane reduction.  B, C, x, dt and the decay of kStage tokens sit in LDS.  The state is read when the rows
+//    log2(NS)-step lane reduction.  B, C, x, dt and the decay of kStage tokens sit in LDS; a stage comes in as 16-byte
+//    pieces, six of them in flight per lane before the first is waited for.  The state is read when the rows
 //    of the launch do not start the sequence and written back after the last row, so a prompt cut into portions, single
 //    decode tokens and a slot that another request held all take one path.
 //  * ssm_post_kernel: gate, grouped norm, weight -> the output projection's input, a workgroup per token.
-//  * ssm_decode_kernel: all of the above for batches of one token per request, a workgroup per (request, head).
+//  * ssm_decode_kernel: all of the above for batches of one token per request whose state is small, a workgroup per request.
 #include "common.h"
 
 namespace semipd {
@@ -75,7 +76,24 @@ __device__ __forceinline__ float ssm_conv_channel(const SsmArgs& a, const T* p, 
 }
 
 // ---------------------------------------------------------------------------------- convolution, silu, step sizes, decays
-template <typename T>
+constexpr int kPrepChannels = 1024;      // channels per workgroup (blockIdx.y walks a token's channels)
+
+// four adjacent elements of the activation type in one access
+template <typename T> __device__ __forceinline__ void load4(const T* p, float (&x)[4]) {
+  if constexpr (sizeof(T) == 2) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    T e;
+    e.v = (uint16_t)(w.x & 0xffffu); x[0] = Elem<T>::to_f(e);
+    e.v = (uint16_t)(w.x >> 16);     x[1] = Elem<T>::to_f(e);
+    e.v = (uint16_t)(w.y & 0xffffu); x[2] = Elem<T>::to_f(e);
+    e.v = (uint16_t)(w.y >> 16);     x[3] = Elem<T>::to_f(e);
+  } else {
+    const float4 w = *reinterpret_cast<const float4*>(p);
+    x[0] = w.x; x[1] = w.y; x[2] = w.z; x[3] = w.w;
+  }
+}
+
+template <typename T, bool VEC4>
 __global__ void __launch_bounds__(256) ssm_prep_kernel(SsmArgs a) {
   const int64_t t = blockIdx.x;
   int b;
@@ -85,12 +103,39 @@ __global__ void __launch_bounds__(256) ssm_prep_kernel(SsmArgs a) {
   const T* p = (const T*)a.p;
   const float* cs = a.conv_state + a.state_indices[b] * a.conv_ld;
   float* w = a.work + t * a.wld;
-  for (int c = threadIdx.x; c < C; c += 256) w[c] = ssm_conv_channel<T>(a, p, cs, first_pos == 0, t, li, c, C);
-  for (int h = threadIdx.x; h < a.H; h += 256) {
-    const float dt = ssm_softplus(Elem<T>::to_f(p[t * a.ld + a.dt_off + h]) + a.dt_bias[h]);
-    w[C + h] = dt;
-    w[C + a.H + h] = expf(-expf(a.a_log[h]) * dt);
+  const int c_lo = blockIdx.y * kPrepChannels;
+  const int c_hi = c_lo + kPrepChannels < C ? c_lo + kPrepChannels : C;
+  const bool fresh = first_pos == 0;
+  if constexpr (VEC4) {
+    // four channels per thread: 8- / 16-byte reads of the inputs and of the state's rows, one 16-byte write
+    const int taps = a.taps;
+    for (int c = c_lo + 4 * threadIdx.x; c < c_hi; c += 1024) {
+      float y[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) y[u] = a.conv_b ? Elem<T>::to_f(((const T*)a.conv_b)[c + u]) : 0.f;
+      const T* cw = (const T*)a.conv_w + (int64_t)c * taps;
+      for (int i = 0; i < taps; ++i) {
+        const int64_t l = li - i;
+        float x[4] = {0.f, 0.f, 0.f, 0.f};
+        if (l >= 0) load4(p + (t - i) * a.ld + a.x_off + c, x);
+        else if (!fresh) {
+          const float4 v = *reinterpret_cast<const float4*>(cs + (int64_t)(taps - 1 + l) * C + c);
+          x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) y[u] += Elem<T>::to_f(cw[u * taps + taps - 1 - i]) * x[u];
+      }
+      *reinterpret_cast<float4*>(w + c) = float4{ssm_silu(y[0]), ssm_silu(y[1]), ssm_silu(y[2]), ssm_silu(y[3])};
+    }
+  } else {
+    for (int c = c_lo + threadIdx.x; c < c_hi; c += 256) w[c] = ssm_conv_channel<T>(a, p, cs, fresh, t, li, c, C);
   }
+  if (blockIdx.y == 0)
+    for (int h = threadIdx.x; h < a.H; h += 256) {
+      const float dt = ssm_softplus(Elem<T>::to_f(p[t * a.ld + a.dt_off + h]) + a.dt_bias[h]);
+      w[C + h] = dt;
+      w[C + a.H + h] = expf(-expf(a.a_log[h]) * dt);
+    }
 }
 
 // ---------------------------------------------------------------------------------- the inputs the next portion looks back at
@@ -125,11 +170,12 @@ __global__ void __launch_bounds__(256) ssm_conv_state_kernel(SsmArgs a) {
 // ---------------------------------------------------------------------------------- the recurrence
 constexpr int kSsmStage = 16;      // tokens whose B, C, x, dt and decay sit in LDS at a time
 
-template <int NPT, int NS>
+template <int NPT, int NS, bool VEC4>
 __global__ void __launch_bounds__(64) ssm_scan_kernel(SsmArgs a) {
   // per staged token: B [NP] | C [NP] | x of the block's columns [COLS] | dt | decay | 2 unused
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int NP = NPT * NS, COLS = 64 / NS, TOK = 2 * NP + COLS + 4;
+  constexpr int NP = NPT * NS, COLS = 64 / NS, TOK = 2 * NP + COLS + 4, TOKU = TOK / 4;
+  constexpr int U = 6;          // 16-byte pieces a lane has in flight while a stage comes in
   const int lane = threadIdx.x;
   const int H = a.H, G = a.G, N = a.N, E = a.E;
   const int eblocks = (E + COLS - 1) / COLS;
@@ -155,20 +201,42 @@ __global__ void __launch_bounds__(64) ssm_scan_kernel(SsmArgs a) {
 #pragma unroll
   for (int i = 0; i < NPT; ++i) S[i] = (first_pos > 0 && e_ok && n0 + i < N) ? st[(int64_t)(n0 + i) * E + e] : 0.f;
   const float dskip = a.d_skip ? a.d_skip[h] : 0.f;
+  // piece u of a staged token: four of B, of C, of the block's x, or (dt, decay, -, -); rows shorter than NP are zero-filled
+  auto piece = [&](const float* w, int u) -> float4 {
+    const float* src;
+    int have;                     // elements of the piece that exist
+    if (u < NP / 4) {
+      src = w + H * E + g * N + 4 * u;
+      have = N - 4 * u;
+    } else if (u < NP / 2) {
+      src = w + H * E + G * N + g * N + 4 * (u - NP / 4);
+      have = N - 4 * (u - NP / 4);
+    } else if (u < NP / 2 + COLS / 4) {
+      src = w + h * E + eb * COLS + 4 * (u - NP / 2);
+      have = E - eb * COLS - 4 * (u - NP / 2);
+    } else {
+      return float4{w[C + h], w[C + H + h], 0.f, 0.f};
+    }
+    if (have <= 0) return float4{0.f, 0.f, 0.f, 0.f};
+    if (VEC4 && have >= 4) return *reinterpret_cast<const float4*>(src);
+    return float4{src[0], have > 1 ? src[1] : 0.f, have > 2 ? src[2] : 0.f, have > 3 ? src[3] : 0.f};
+  };
   for (int64_t s0 = 0; s0 < n; s0 += kSsmStage) {
     const int cnt = (int)((n - s0) < kSsmStage ? (n - s0) : kSsmStage);
+    const int total = cnt * TOKU;
+    const float* w0 = a.work + (t0 + s0) * a.wld;
     __syncthreads();
-    for (int k = 0; k < cnt; ++k) {
-      const float* w = a.work + (t0 + s0 + k) * a.wld;
-      float* l = lds + k * TOK;
-      for (int i = lane; i < NP; i += 64) {
-        l[i] = i < N ? w[H * E + g * N + i] : 0.f;
-        l[NP + i] = i < N ? w[H * E + G * N + g * N + i] : 0.f;
+    for (int base = 0; base < total; base += 64 * U) {
+      float4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int it = base + u * 64 + lane;
+        v[u] = it < total ? piece(w0 + (int64_t)(it / TOKU) * a.wld, it % TOKU) : float4{0.f, 0.f, 0.f, 0.f};
       }
-      if (lane < COLS) l[2 * NP + lane] = (eb * COLS + lane < E) ? w[h * E + eb * COLS + lane] : 0.f;
-      if (lane == 0) {
-        l[2 * NP + COLS] = w[C + h];
-        l[2 * NP + COLS + 1] = w[C + H + h];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int it = base + u * 64 + lane;
+        if (it < total) *reinterpret_cast<float4*>(lds + 4 * it) = v[u];
       }
     }
     __syncthreads();
@@ -337,17 +405,27 @@ extern "C" int semipd_state_space(const void* proj, int64_t ld, int64_t z_off, i
   }
   SEMIPD_CHECK_ARG(work && work_ld >= semipd_state_space_work_width(num_heads, groups, state_size, v_dim), SEMIPD_EINVAL,
                    "state_space: the work rows are missing or too short");
-  SEMIPD_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL((ssm_prep_kernel<T>), dim3((unsigned)num_tokens), dim3(256), 0, s, a));
+  const unsigned cblocks = (unsigned)((C + kPrepChannels - 1) / kPrepChannels);
+  // four channels per thread: every row and column range starts on a multiple of four elements
+  const bool prep4 = C % 4 == 0 && x_off % 4 == 0 && ld % 4 == 0 && work_ld % 4 == 0 && (taps == 1 || conv_ld % 4 == 0) &&
+                     ((uintptr_t)proj % 16) == 0 && aligned16(work) && (taps == 1 || aligned16(conv_state));
+  SEMIPD_DISPATCH_DTYPE(dtype, T, {
+    if (prep4) hipLaunchKernelGGL((ssm_prep_kernel<T, true>), dim3((unsigned)num_tokens, cblocks), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((ssm_prep_kernel<T, false>), dim3((unsigned)num_tokens, cblocks), dim3(256), 0, s, a);
+  });
   if (taps > 1) {
     const dim3 grid((unsigned)((C + 255) / 256), (unsigned)batch);
     SEMIPD_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL((ssm_conv_state_kernel<T>), grid, dim3(256), 0, s, a));
   }
+  // 16-byte staging reads: B, C and x of a token start on multiples of four floats
+  const bool scan4 = work_ld % 4 == 0 && aligned16(work) && inner % 4 == 0 && state_size % 4 == 0 && v_dim % 4 == 0;
 #define SEMIPD_SSM_SCAN(NPT, NS)                                                                                              \
   do {                                                                                                                        \
     constexpr int cols = 64 / NS;                                                                                             \
     const unsigned blocks = (unsigned)(batch * num_heads * ((v_dim + cols - 1) / cols));                                      \
     const size_t bytes = (size_t)kSsmStage * (2 * NPT * NS + cols + 4) * sizeof(float);                                       \
-    hipLaunchKernelGGL((ssm_scan_kernel<NPT, NS>), dim3(blocks), dim3(64), bytes, s, a);                                      \
+    if (scan4) hipLaunchKernelGGL((ssm_scan_kernel<NPT, NS, true>), dim3(blocks), dim3(64), bytes, s, a);                     \
+    else hipLaunchKernelGGL((ssm_scan_kernel<NPT, NS, false>), dim3(blocks), dim3(64), bytes, s, a);                          \
   } while (0)
   if (state_size <= 16) SEMIPD_SSM_SCAN(16, 1);
   else if (state_size <= 32) SEMIPD_SSM_SCAN(32, 1);

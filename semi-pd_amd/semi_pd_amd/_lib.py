@@ -182,7 +182,7 @@ _SIGNATURES = {
     "semipd_qk_norm_rope_kv_store": [_vp, _i64, _i64, _i32, _i32, _i32, _i32, _i64, _i64, _vp, _vp, _f32, _vp, _vp, _i32, _i32, _f32,
                                      _vp, _vp, _vp, _vp, _i32, _vp],
     "semipd_shared_value_attention": [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32,
-                                      _i32, _i32, _f32, _i32, _i32, _vp],
+                                      _i32, _i32, _f32, _i32, _vp, _i32, _i32, _vp],
     "semipd_talk_mix": [_vp, _i64, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
     "semipd_state_space_work_width": [_i32, _i32, _i32, _i32],
     "semipd_state_space": [_vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _vp, _i64, _vp, _i64, _vp, _i64,

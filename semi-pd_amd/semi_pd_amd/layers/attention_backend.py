@@ -343,9 +343,15 @@ class HipAttnBackend(AttentionBackend):
         G = layer.tp_k_head_num
         o = torch.empty((T, layer.tp_q_head_num * G * layer.v_head_dim), dtype=q.dtype, device=q.device)
         pool = forward_batch.token_to_kv_pool
+        n_splits = 1
         if forward_batch.forward_mode.is_decode():
             q_start = q_len = None
             max_q = 1
+            # a decode batch is (requests x key/value heads x groups of 16 heads) workgroups: below two per CU the keys of a
+            # request are shared out over several, about 128 keys each at least (as forward_latent does)
+            wgs = T * G * ((layer.tp_q_head_num // G + 15) // 16)
+            n_splits = max(1, min(16, (2 * max(1, self.num_cus)) // max(wgs, 1), self._decode_len_bound // 128))
+            n_splits = int(os.environ.get("SEMIPD_SHARED_VALUE_DECODE_SPLITS", n_splits))
         else:
             q_start, q_len = forward_batch.extend_start_loc, forward_batch.extend_seq_lens
             max_q = max(forward_batch.extend_seq_lens_cpu)
@@ -353,7 +359,8 @@ class HipAttnBackend(AttentionBackend):
         t0 = kt.start() if kt else None
         ops.shared_value_attention_fwd(q, o, pool.get_key_buffer(layer.layer_id), pool.get_value_buffer(layer.layer_id),
                                        self.req_to_token, forward_batch.req_pool_indices, forward_batch.seq_lens, q_start, q_len,
-                                       max_q, layer.scaling, form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")))
+                                       max_q, layer.scaling, form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")),
+                                       n_splits=n_splits)
         if kt:
             kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
         return o

@@ -1917,10 +1917,12 @@ def qk_norm_rope_kv_store(qkv: torch.Tensor, num_q_heads: int, num_kv_heads: int
 def shared_value_attention_fwd(q: torch.Tensor, out: torch.Tensor, k_buffer: torch.Tensor, v_buffer: torch.Tensor,
                                req_to_token: torch.Tensor, req_pool_indices: torch.Tensor, seq_lens: torch.Tensor,
                                q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor], max_q_len: int, sm_scale: float,
-                               form: int = 0) -> None:
+                               form: int = 0, n_splits: int = 1) -> None:
     """Causal softmax attention over the paged pools in which every query head's weights are applied to the values of ALL
     key/value heads: q [T, H * D], keys [N, G, D] (head h reads key head h / (H / G)), values [N, G, E] read as one row of
-    G * E elements, out [T, H * G * E].  Batch description as in local_attention_fwd (csrc/local_attention.hip)."""
+    G * E elements, out [T, H * G * E].  Batch description as in local_attention_fwd (csrc/local_attention.hip).
+    n_splits > 1: a decode batch whose requests' keys are shared out over that many workgroups each (the matrix-core decode
+    form; other forms ignore it)."""
     T = q.shape[0]
     G, D = k_buffer.shape[1], k_buffer.shape[2]
     row = v_buffer.shape[1] * v_buffer.shape[2]
@@ -1935,10 +1937,12 @@ def shared_value_attention_fwd(q: torch.Tensor, out: torch.Tensor, k_buffer: tor
         raise RuntimeError("shared_value_attention_fwd: req_to_token int32, req_pool_indices / seq_lens int64")
     B = req_pool_indices.shape[0]
     _batch_rows("shared_value_attention_fwd", T, B, q_start, q_len)
+    n_splits = int(n_splits) if (q_start is None and q.dtype != torch.float32) else 1
+    partial = torch.empty((T, H, n_splits, row + 2), dtype=torch.float32, device=q.device) if n_splits > 1 else None
     check(_lib.load().semipd_shared_value_attention(ptr(q), q.stride(0), ptr(out), out.stride(0), ptr(k_buffer), ptr(v_buffer),
                                                     ptr(req_to_token), req_to_token.stride(0), ptr(req_pool_indices), ptr(seq_lens),
                                                     ptr(q_start), ptr(q_len), B, T, int(max_q_len), H, G, D, row, float(sm_scale),
-                                                    int(form), dtype_code(q.dtype), current_stream(q.device)),
+                                                    n_splits, ptr(partial), int(form), dtype_code(q.dtype), current_stream(q.device)),
           "shared_value_attention")
 
 

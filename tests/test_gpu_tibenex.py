@@ -241,12 +241,14 @@ def test_attention_over_shared_values_with_mixed_heads(dtype, form, H, G, D, E):
     # a decode batch: one more token each
     lens1 = [n + 1 for n in lens]
     q1 = torch.stack([qs[b][lens[b]] for b in range(4)]).view(4, H * D).to(DEV)
-    parts = torch.empty(4, H * G * E, dtype=dtype, device=DEV)
-    ops.shared_value_attention_fwd(q1, parts, kp, vp, r2t, rp, torch.tensor(lens1, device=DEV), None, None, 1, scale, form=form)
-    out = ops.talk_mix(parts, talk.to(DEV), G).float().cpu().view(4, H, E)
-    for b in range(4):
-        want = _talking_truth(qs[b][lens[b]: lens[b] + 1], ks[b], vs[b], talk, scale)
-        torch.testing.assert_close(out[b: b + 1], want, **tol)
+    for n_splits in (1, 3):                                    # (the keys of a request shared out over three workgroups)
+        parts = torch.empty(4, H * G * E, dtype=dtype, device=DEV)
+        ops.shared_value_attention_fwd(q1, parts, kp, vp, r2t, rp, torch.tensor(lens1, device=DEV), None, None, 1, scale, form=form,
+                                       n_splits=n_splits)
+        out = ops.talk_mix(parts, talk.to(DEV), G).float().cpu().view(4, H, E)
+        for b in range(4):
+            want = _talking_truth(qs[b][lens[b]: lens[b] + 1], ks[b], vs[b], talk, scale)
+            torch.testing.assert_close(out[b: b + 1], want, **tol)
 
 
 # ----------------------------------------------------------------------------------------------- state-space recurrence

@@ -577,7 +577,7 @@ TIBENEX_SIZES = {
                      sheads=128, svdim=64, state=128, groups=8, ff=14336, vocab=32000),
     "3b-layer": dict(hidden=3072, heads=24, dim=64, rot=64, vdim=128, rank=192, qrank=1024, theads=24, tkv=2, tdim=128, tvdim=128,
                      sheads=96, svdim=64, state=128, groups=8, ff=8192, vocab=32000),
-    "1b-layer": dict(hidden=2048, heads=32, dim=32, rot=32, vdim=64, rank=96, qrank=768, theads=32, tkv=4, tdim=64, tvdim=64,
+    "1b-layer": dict(hidden=2048, heads=32, dim=32, rot=32, vdim=64, rank=96, qrank=768, theads=32, tkv=2, tdim=64, tvdim=64,
                      sheads=64, svdim=64, state=64, groups=8, ff=8192, vocab=32000),
 }
 
@@ -679,8 +679,10 @@ def _tibenex_kernel_pairs(s, pz, dev):
     parts2 = torch.empty(B2, H * G * E, device=dev, dtype=dt)
     o2 = torch.empty(B2, H * E, device=dev, dtype=dt)
 
+    tsplits = max(1, min(16, 512 // (B2 * G * ((H // G + 15) // 16)), C // 128))     # HipAttnBackend.forward_shared_values' rule on 256 CUs
+
     def talking_decode():
-        ops.shared_value_attention_fwd(q2, parts2, kp, vp, r2t2, rows2, lens2, None, None, 1, D ** -0.5)
+        ops.shared_value_attention_fwd(q2, parts2, kp, vp, r2t2, rows2, lens2, None, None, 1, D ** -0.5, n_splits=tsplits)
         ops.talk_mix(parts2, talk, G, out=o2)
 
     t_new = _timed(talking_decode)
@@ -689,7 +691,7 @@ def _tibenex_kernel_pairs(s, pz, dev):
     ol = torch.empty(B2, pH * pR, device=dev, dtype=dt)
     splits = max(1, min(16, 512 // (B2 * ((pH + 15) // 16)), C // 128))
     t_old = _timed(lambda: ops.latent_attention_fwd(ql, ol, pool2, pR, r2t2, rows2, lens2, None, None, 1, 0.1, sink, n_splits=splits))
-    out.append((f"decode attention, {B2} requests at {C} tokens, {G} key/value heads of {D} / {E}, + the mix of the heads (like: every latent "
+    out.append((f"decode attention, {B2} requests at {C} tokens, {G} key/value heads of {D} / {E}, {tsplits} workgroups share a request's keys, + merge, + the mix of the heads (like: every latent "
                 f"row of {pR} + {pP} once for all {pH} heads, {splits} workgroups share a request's keys, + merge)",
                 rec(t_new, nbytes=B2 * G * (D + E) * 2.0 * C), rec(t_old, nbytes=B2 * (pR + pP) * 2.0 * C)))
     # ---- the recurrences: a prompt batch and a decode batch ----------------------------------------------------------------
