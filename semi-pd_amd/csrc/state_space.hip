@@ -8,13 +8,14 @@
 // then y * silu(z), an RMS norm over each of `norm_groups` equal parts of the row, times a weight.  Everything behind the
 // projection GEMM is fp32 whatever the activation type.
 //
-//  * ssm_prep_kernel: a workgroup per (token, 1024 channels), four channels per thread where alignment allows: convolution + bias + silu of the token's x | B | C channels (inputs in front
+//  * ssm_prep_kernel: a workgroup per (tile of 32 tokens -- one token in small batches --, 1024 channels), four channels per
+//    thread with their taps in registers where alignment allows: convolution + bias + silu of the token's x | B | C channels (inputs in front
 //    of the portion come from the state row), dt and the decay -> an fp32 work row per token.
 //  * ssm_conv_state_kernel: the last taps - 1 inputs of the portion (shifted in behind what the row held) -> state row.
 //  * ssm_scan_kernel: ONE WAVE per (request, head, block of 64 / NS columns of S); a column of S lives in the registers of NS
 //    adjacent lanes, NPT rows each, so a step is one multiply-add per register for the update, one for the read-out, and a
-//    log2(NS)-step lane reduction.  B, C, x, dt and the decay of kStage tokens sit in LDS; a stage comes in as 16-byte
-//    pieces, six of them in flight per lane before the first is waited for.  The state is read when the rows
+//    log2(NS)-step lane reduction.  B, C, x, dt and the decay of kStage tokens sit in LDS; the next stage's 16-byte pieces are
+//    fetched into registers while a stage is multiplied and go into the other half of the LDS buffer behind it.  The state is read when the rows
 //    of the launch do not start the sequence and written back after the last row, so a prompt cut into portions, single
 //    decode tokens and a slot that another request held all take one path.
 //  * ssm_post_kernel: gate, grouped norm, weight -> the output projection's input, a workgroup per token.
@@ -93,49 +94,68 @@ template <typename T> __device__ __forceinline__ void load4(const T* p, float (&
   }
 }
 
+constexpr int kPrepMaxTaps = 8;          // taps whose weights the four-channel form keeps in registers
+constexpr int kPrepTile = 32;            // tokens a workgroup of a prompt batch walks with them
+
 template <typename T, bool VEC4>
-__global__ void __launch_bounds__(256) ssm_prep_kernel(SsmArgs a) {
-  const int64_t t = blockIdx.x;
-  int b;
-  int64_t li, n, first_pos;
-  if (!ssm_locate(a, t, b, li, n, first_pos)) return;
+__global__ void __launch_bounds__(256) ssm_prep_kernel(SsmArgs a, int tile) {
   const int C = a.H * a.E + 2 * a.G * a.N;
   const T* p = (const T*)a.p;
-  const float* cs = a.conv_state + a.state_indices[b] * a.conv_ld;
-  float* w = a.work + t * a.wld;
   const int c_lo = blockIdx.y * kPrepChannels;
   const int c_hi = c_lo + kPrepChannels < C ? c_lo + kPrepChannels : C;
-  const bool fresh = first_pos == 0;
-  if constexpr (VEC4) {
-    // four channels per thread: 8- / 16-byte reads of the inputs and of the state's rows, one 16-byte write
-    const int taps = a.taps;
-    for (int c = c_lo + 4 * threadIdx.x; c < c_hi; c += 1024) {
-      float y[4];
+  const int taps = a.taps;
+  // four channels per thread (8- / 16-byte reads of the inputs and of the state's rows, one 16-byte write), their taps and
+  // bias in registers for all tokens of the tile
+  const int c4 = c_lo + 4 * threadIdx.x;
+  const bool mine = VEC4 && c4 < c_hi;
+  float wt[kPrepMaxTaps][4], bias[4] = {0.f, 0.f, 0.f, 0.f};
+  if (mine) {
+    const T* cw = (const T*)a.conv_w + (int64_t)c4 * taps;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) y[u] = a.conv_b ? Elem<T>::to_f(((const T*)a.conv_b)[c + u]) : 0.f;
-      const T* cw = (const T*)a.conv_w + (int64_t)c * taps;
-      for (int i = 0; i < taps; ++i) {
-        const int64_t l = li - i;
-        float x[4] = {0.f, 0.f, 0.f, 0.f};
-        if (l >= 0) load4(p + (t - i) * a.ld + a.x_off + c, x);
-        else if (!fresh) {
-          const float4 v = *reinterpret_cast<const float4*>(cs + (int64_t)(taps - 1 + l) * C + c);
-          x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
-        }
+    for (int i = 0; i < kPrepMaxTaps; ++i)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) y[u] += Elem<T>::to_f(cw[u * taps + taps - 1 - i]) * x[u];
-      }
-      *reinterpret_cast<float4*>(w + c) = float4{ssm_silu(y[0]), ssm_silu(y[1]), ssm_silu(y[2]), ssm_silu(y[3])};
-    }
-  } else {
-    for (int c = c_lo + threadIdx.x; c < c_hi; c += 256) w[c] = ssm_conv_channel<T>(a, p, cs, fresh, t, li, c, C);
+      for (int u = 0; u < 4; ++u) wt[i][u] = i < taps ? Elem<T>::to_f(cw[u * taps + taps - 1 - i]) : 0.f;      // i tokens back
+    if (a.conv_b)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) bias[u] = Elem<T>::to_f(((const T*)a.conv_b)[c4 + u]);
   }
-  if (blockIdx.y == 0)
-    for (int h = threadIdx.x; h < a.H; h += 256) {
-      const float dt = ssm_softplus(Elem<T>::to_f(p[t * a.ld + a.dt_off + h]) + a.dt_bias[h]);
-      w[C + h] = dt;
-      w[C + a.H + h] = expf(-expf(a.a_log[h]) * dt);
+  for (int tt = 0; tt < tile; ++tt) {
+    const int64_t t = (int64_t)blockIdx.x * tile + tt;
+    if (t >= a.num_tokens) break;
+    int b;
+    int64_t li, n, first_pos;
+    if (!ssm_locate(a, t, b, li, n, first_pos)) continue;
+    const float* cs = a.conv_state + a.state_indices[b] * a.conv_ld;
+    float* w = a.work + t * a.wld;
+    const bool fresh = first_pos == 0;
+    if constexpr (VEC4) {
+      if (mine) {
+        float y[4] = {bias[0], bias[1], bias[2], bias[3]};
+#pragma unroll
+        for (int i = 0; i < kPrepMaxTaps; ++i) {
+          if (i >= taps) break;
+          const int64_t l = li - i;
+          float x[4] = {0.f, 0.f, 0.f, 0.f};
+          if (l >= 0) load4(p + (t - i) * a.ld + a.x_off + c4, x);
+          else if (!fresh) {
+            const float4 v = *reinterpret_cast<const float4*>(cs + (int64_t)(taps - 1 + l) * C + c4);
+            x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) y[u] += wt[i][u] * x[u];
+        }
+        *reinterpret_cast<float4*>(w + c4) = float4{ssm_silu(y[0]), ssm_silu(y[1]), ssm_silu(y[2]), ssm_silu(y[3])};
+      }
+    } else {
+      for (int c = c_lo + threadIdx.x; c < c_hi; c += 256) w[c] = ssm_conv_channel<T>(a, p, cs, fresh, t, li, c, C);
     }
+    if (blockIdx.y == 0)
+      for (int h = threadIdx.x; h < a.H; h += 256) {
+        const float dt = ssm_softplus(Elem<T>::to_f(p[t * a.ld + a.dt_off + h]) + a.dt_bias[h]);
+        w[C + h] = dt;
+        w[C + a.H + h] = expf(-expf(a.a_log[h]) * dt);
+      }
+  }
 }
 
 // ---------------------------------------------------------------------------------- the inputs the next portion looks back at
@@ -168,14 +188,16 @@ __global__ void __launch_bounds__(256) ssm_conv_state_kernel(SsmArgs a) {
 }
 
 // ---------------------------------------------------------------------------------- the recurrence
-constexpr int kSsmStage = 16;      // tokens whose B, C, x, dt and decay sit in LDS at a time
+constexpr int kSsmStage = 8;       // tokens of a stage: their B, C, x, dt and decay sit in LDS, the next stage's in registers
 
 template <int NPT, int NS, bool VEC4>
 __global__ void __launch_bounds__(64) ssm_scan_kernel(SsmArgs a) {
-  // per staged token: B [NP] | C [NP] | x of the block's columns [COLS] | dt | decay | 2 unused
+  // per staged token: B [NP] | C [NP] | x of the block's columns [COLS] | dt | decay | 2 unused.  B and C are cut into the NS
+  // slices that the lanes of a column read, each slice followed by 4 unused floats: the 16-byte reads of the NS lanes then
+  // fall into different banks (slices of 32 floats alone would put lanes 0 and 2 on the same ones)
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int NP = NPT * NS, COLS = 64 / NS, TOK = 2 * NP + COLS + 4, TOKU = TOK / 4;
-  constexpr int U = 6;          // 16-byte pieces a lane has in flight while a stage comes in
+  constexpr int SEG = NS > 1 ? NPT + 4 : NPT, NP = SEG * NS, COLS = 64 / NS, TOK = 2 * NP + COLS + 4, TOKU = TOK / 4;
+  constexpr int U = (kSsmStage * TOKU + 63) / 64;          // 16-byte pieces of a stage per lane
   const int lane = threadIdx.x;
   const int H = a.H, G = a.G, N = a.N, E = a.E;
   const int eblocks = (E + COLS - 1) / COLS;
@@ -205,12 +227,12 @@ __global__ void __launch_bounds__(64) ssm_scan_kernel(SsmArgs a) {
   auto piece = [&](const float* w, int u) -> float4 {
     const float* src;
     int have;                     // elements of the piece that exist
-    if (u < NP / 4) {
-      src = w + H * E + g * N + 4 * u;
-      have = N - 4 * u;
-    } else if (u < NP / 2) {
-      src = w + H * E + G * N + g * N + 4 * (u - NP / 4);
-      have = N - 4 * (u - NP / 4);
+    if (u < NP / 2) {
+      const int pos = 4 * (u < NP / 4 ? u : u - NP / 4), off = pos % SEG;
+      if (off >= NPT) return float4{0.f, 0.f, 0.f, 0.f};                 // the gap behind a slice
+      const int i = (pos / SEG) * NPT + off;                               // row of the state
+      src = w + H * E + (u < NP / 4 ? 0 : G * N) + g * N + i;
+      have = N - i;
     } else if (u < NP / 2 + COLS / 4) {
       src = w + h * E + eb * COLS + 4 * (u - NP / 2);
       have = E - eb * COLS - 4 * (u - NP / 2);
@@ -221,34 +243,44 @@ __global__ void __launch_bounds__(64) ssm_scan_kernel(SsmArgs a) {
     if (VEC4 && have >= 4) return *reinterpret_cast<const float4*>(src);
     return float4{src[0], have > 1 ? src[1] : 0.f, have > 2 ? src[2] : 0.f, have > 3 ? src[3] : 0.f};
   };
-  for (int64_t s0 = 0; s0 < n; s0 += kSsmStage) {
+  // A stage's pieces are fetched into registers while the stage in front of it is multiplied, and put into the other half
+  // of the LDS buffer behind it: the loads of HBM rows are in flight during the arithmetic.
+  float4 v[U];
+  auto fetch = [&](int64_t s0) {
     const int cnt = (int)((n - s0) < kSsmStage ? (n - s0) : kSsmStage);
     const int total = cnt * TOKU;
     const float* w0 = a.work + (t0 + s0) * a.wld;
-    __syncthreads();
-    for (int base = 0; base < total; base += 64 * U) {
-      float4 v[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int it = base + u * 64 + lane;
-        v[u] = it < total ? piece(w0 + (int64_t)(it / TOKU) * a.wld, it % TOKU) : float4{0.f, 0.f, 0.f, 0.f};
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int it = base + u * 64 + lane;
-        if (it < total) *reinterpret_cast<float4*>(lds + 4 * it) = v[u];
-      }
+    for (int u = 0; u < U; ++u) {
+      const int it = u * 64 + lane;
+      v[u] = it < total ? piece(w0 + (int64_t)(it / TOKU) * a.wld, it % TOKU) : float4{0.f, 0.f, 0.f, 0.f};
     }
-    __syncthreads();
+  };
+  auto stash = [&](float* buf) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int it = u * 64 + lane;
+      if (it < kSsmStage * TOKU) *reinterpret_cast<float4*>(buf + 4 * it) = v[u];
+    }
+  };
+  fetch(0);
+  stash(lds);
+  __syncthreads();
+  int half = 0;
+  for (int64_t s0 = 0; s0 < n; s0 += kSsmStage) {
+    const int cnt = (int)((n - s0) < kSsmStage ? (n - s0) : kSsmStage);
+    const bool more = s0 + kSsmStage < n;
+    if (more) fetch(s0 + kSsmStage);
+    const float* stage = lds + half * (kSsmStage * TOK);
     for (int k = 0; k < cnt; ++k) {
-      const float* l = lds + k * TOK;
+      const float* l = stage + k * TOK;
       const float xv = l[2 * NP + col], dtv = l[2 * NP + COLS], dec = l[2 * NP + COLS + 1];
       const float dx = dtv * xv;
       float y = 0.f;
 #pragma unroll
       for (int i = 0; i < NPT; i += 4) {
-        const float4 bv = *reinterpret_cast<const float4*>(l + n0 + i);
-        const float4 cv = *reinterpret_cast<const float4*>(l + NP + n0 + i);
+        const float4 bv = *reinterpret_cast<const float4*>(l + ns * SEG + i);
+        const float4 cv = *reinterpret_cast<const float4*>(l + NP + ns * SEG + i);
         S[i] = dec * S[i] + bv.x * dx;         y += S[i] * cv.x;
         S[i + 1] = dec * S[i + 1] + bv.y * dx; y += S[i + 1] * cv.y;
         S[i + 2] = dec * S[i + 2] + bv.z * dx; y += S[i + 2] * cv.z;
@@ -259,6 +291,9 @@ __global__ void __launch_bounds__(64) ssm_scan_kernel(SsmArgs a) {
       if (NS >= 8) y += __shfl_xor(y, 4, 64);
       if (ns == 0 && e_ok) a.work[(t0 + s0 + k) * a.wld + h * E + e] = y + dskip * xv;
     }
+    half ^= 1;
+    if (more) stash(lds + half * (kSsmStage * TOK));
+    __syncthreads();
   }
   if (e_ok) {
 #pragma unroll
@@ -408,10 +443,14 @@ extern "C" int semipd_state_space(const void* proj, int64_t ld, int64_t z_off, i
   const unsigned cblocks = (unsigned)((C + kPrepChannels - 1) / kPrepChannels);
   // four channels per thread: every row and column range starts on a multiple of four elements
   const bool prep4 = C % 4 == 0 && x_off % 4 == 0 && ld % 4 == 0 && work_ld % 4 == 0 && (taps == 1 || conv_ld % 4 == 0) &&
-                     ((uintptr_t)proj % 16) == 0 && aligned16(work) && (taps == 1 || aligned16(conv_state));
+                     ((uintptr_t)proj % 16) == 0 && aligned16(work) && (taps == 1 || aligned16(conv_state)) &&
+                     aligned16(conv_w) && taps <= kPrepMaxTaps;
+  // a prompt batch: a workgroup walks a tile of tokens with its channels' taps in registers; one row per request: a token each
+  const int tile = (q_start != nullptr && prep4 && num_tokens >= 8 * kPrepTile) ? kPrepTile : 1;
+  const dim3 pgrid((unsigned)((num_tokens + tile - 1) / tile), cblocks);
   SEMIPD_DISPATCH_DTYPE(dtype, T, {
-    if (prep4) hipLaunchKernelGGL((ssm_prep_kernel<T, true>), dim3((unsigned)num_tokens, cblocks), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((ssm_prep_kernel<T, false>), dim3((unsigned)num_tokens, cblocks), dim3(256), 0, s, a);
+    if (prep4) hipLaunchKernelGGL((ssm_prep_kernel<T, true>), pgrid, dim3(256), 0, s, a, tile);
+    else hipLaunchKernelGGL((ssm_prep_kernel<T, false>), pgrid, dim3(256), 0, s, a, tile);
   });
   if (taps > 1) {
     const dim3 grid((unsigned)((C + 255) / 256), (unsigned)batch);
@@ -423,7 +462,7 @@ extern "C" int semipd_state_space(const void* proj, int64_t ld, int64_t z_off, i
   do {                                                                                                                        \
     constexpr int cols = 64 / NS;                                                                                             \
     const unsigned blocks = (unsigned)(batch * num_heads * ((v_dim + cols - 1) / cols));                                      \
-    const size_t bytes = (size_t)kSsmStage * (2 * NPT * NS + cols + 4) * sizeof(float);                                       \
+    const size_t bytes = 2 * (size_t)kSsmStage * (2 * (NS > 1 ? NPT + 4 : NPT) * NS + cols + 4) * sizeof(float);              \
     if (scan4) hipLaunchKernelGGL((ssm_scan_kernel<NPT, NS, true>), dim3(blocks), dim3(64), bytes, s, a);                     \
     else hipLaunchKernelGGL((ssm_scan_kernel<NPT, NS, false>), dim3(blocks), dim3(64), bytes, s, a);                          \
   } while (0)
